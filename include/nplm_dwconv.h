@@ -1,0 +1,114 @@
+/*
+ * nplm_dwconv.h — C ABI of libnplm_dwconv.so: variable-length depthwise 1-D convolution over
+ * packed sequences, forward and backward, for AMD MI355X (gfx950).
+ *
+ * The operator
+ * ------------
+ *   x, y, dy, dx : [T, C] row-major, contiguous (packed tokens x channels)
+ *   w            : [C, K] row-major, K odd, P = (K-1)/2 (centred "same" padding)
+ *   b            : [C] or NULL
+ *   cu           : int32 [S+1], cu[0] = 0, non-decreasing, cu[S] = T. Sequence i owns rows
+ *                  [cu[i], cu[i+1]). Zero-length sequences (cu[i] == cu[i+1]) are legal anywhere.
+ *
+ *   y [t,c] = b[c] + sum_k w[c,k] * x [t+k-P, c] * [s(t) <= t+k-P < e(t)]
+ *   dx[t,c] =        sum_k w[c,k] * dy[t-k+P, c] * [s(t) <= t-k+P < e(t)]
+ *   dw[c,k] = sum_t dy[t,c] * x[t+k-P, c] * [s(t) <= t+k-P < e(t)]
+ *   db[c]   = sum_t dy[t,c]
+ *   with [s(t), e(t)) the cu interval that contains row t. Taps never cross a sequence boundary
+ *   (masked by selection, so a NaN/Inf in one sequence cannot reach another).
+ *
+ * Where this sits in the reference (peymanvahidi/nanoplm 0.1.6): the reference snapshot holds no
+ * convolution; the ABI binds at the call site a conv module would occupy on the packed path,
+ * src/nanoplm/pretraining/models/modern_bert/modeling.py:421-439 (encoder layer over x:[T,hidden]
+ * with cu_seqlens), with the data contract of src/nanoplm/pretraining/collator.py:308-325
+ * (cu_seqlens int32) and :405-458 (fixed-length cu_seqlens with trailing zero-length entries), and
+ * the flat (total_tokens, hidden) layout of modeling.py:339,464. Each entry point below names the
+ * autograd stage of that module it implements.
+ *
+ * Conventions
+ * -----------
+ *  - All pointers are DEVICE pointers owned by the caller. The library never allocates or frees
+ *    device memory, keeps no pointer after return and has no mutable global state.
+ *  - All work is enqueued asynchronously on `stream` (a hipStream_t passed as void*; NULL = the
+ *    null stream). cu is read on the device: no host synchronisation.
+ *  - Launch geometry depends only on (T, C, K, dtypes), never on timing: results are
+ *    run-to-run bit-identical (no floating-point atomics anywhere).
+ *  - Return value: 0 on success; < 0 an NPLM_DWCONV_E* argument error (nothing was launched);
+ *    > 0 a hipError_t from a launch.
+ *  - Preconditions NOT checked on the fast path (they would need a device read-back):
+ *    cu[0] == 0, cu non-decreasing, cu[S] == T. Violations never cause out-of-bounds accesses
+ *    (cu is only used to mask taps); rows outside [cu[0], cu[S]) are treated as one extra
+ *    sequence on that side. nplm_dwconv_check_cu() verifies them with a read-back.
+ */
+#ifndef NPLM_DWCONV_H
+#define NPLM_DWCONV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types for act_dtype / w_dtype */
+#define NPLM_DWCONV_F32  0
+#define NPLM_DWCONV_BF16 1
+
+/* argument errors (returned negated: -NPLM_DWCONV_E...) */
+#define NPLM_DWCONV_ENULL      1  /* a required pointer is NULL */
+#define NPLM_DWCONV_ESHAPE     2  /* T < 0, T > 2^31 - 2^20 - 1, C < 1, S < 0, or C*K too large */
+#define NPLM_DWCONV_EKSIZE     3  /* K < 1, K even, or K > NPLM_DWCONV_MAX_K */
+#define NPLM_DWCONV_EDTYPE     4  /* unknown act_dtype / w_dtype */
+#define NPLM_DWCONV_EALIGN     5  /* activation pointer not aligned to its element size */
+#define NPLM_DWCONV_EWORKSPACE 6  /* workspace NULL, misaligned (256 B) or smaller than required */
+#define NPLM_DWCONV_ECU        7  /* check_cu: cu[0] != 0, cu decreasing, or cu[S] != T */
+
+#define NPLM_DWCONV_MAX_K 255
+
+/* Library version: major*10000 + minor*100 + patch. */
+int nplm_dwconv_version(void);
+
+/* Text for a return code of any entry point (argument errors and hipError_t values). */
+const char* nplm_dwconv_strerror(int code);
+
+/*
+ * Forward: y = conv(x; w, b) per sequence.
+ * Implements the module's forward at modeling.py:421-439 (x:[T,C] with cu_seqlens).
+ * x, y: act_dtype; w, b: w_dtype (b may be NULL). bf16 activations are accumulated in fp32 and
+ * rounded once (nearest-even) on store. T == 0 is a no-op.
+ */
+int nplm_dwconv_fwd(const void* x, const int32_t* cu, const void* w, const void* b, void* y,
+                    int64_t T, int32_t C, int32_t K, int32_t S,
+                    int32_t act_dtype, int32_t w_dtype, void* stream);
+
+/*
+ * Bytes of device workspace nplm_dwconv_bwd needs for these sizes (fp32 partial sums of dw/db,
+ * one slab per token-range block). Pure host arithmetic; 0 is returned for invalid sizes.
+ */
+size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype);
+
+/*
+ * Backward: dx (act_dtype), dw [C,K] and db [C] (always fp32, fully overwritten) from x, dy.
+ * Implements what autograd runs for the same module during loss.backward()
+ * (src/nanoplm/pretraining/pure_pipeline.py:739-742). One fused pass reads x and dy once and
+ * writes dx once; dw/db partials go to `workspace` (256-byte aligned, at least
+ * nplm_dwconv_bwd_workspace_bytes() bytes, contents irrelevant on entry) and a second small
+ * kernel sums them in a fixed order. dx, dw or db may each be NULL only if all of the outputs
+ * it belongs with are skipped: dx == NULL skips dx; dw == NULL && db == NULL skips the
+ * reductions (workspace may then be NULL). T == 0 zero-fills dw and db.
+ */
+int nplm_dwconv_bwd(const void* x, const void* dy, const int32_t* cu, const void* w,
+                    void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,
+                    int64_t T, int32_t C, int32_t K, int32_t S,
+                    int32_t act_dtype, int32_t w_dtype, void* stream);
+
+/*
+ * Debug helper: copies cu to the host (synchronises `stream`) and verifies the preconditions.
+ * Returns 0, -NPLM_DWCONV_ECU, another argument error, or a hipError_t.
+ */
+int nplm_dwconv_check_cu(const int32_t* cu, int32_t S, int64_t T, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NPLM_DWCONV_H */

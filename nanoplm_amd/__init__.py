@@ -1,0 +1,12 @@
+"""nanoplm_amd: MI355X-native varlen depthwise 1-D convolution for nanoPLM's packed conv path."""
+from .dwconv import (  # noqa: F401
+    VarlenDWConv1d,
+    VarlenDWConv1dFunction,
+    bwd_workspace_bytes,
+    check_cu_seqlens,
+    varlen_dwconv,
+    varlen_dwconv_bwd,
+    varlen_dwconv_fwd,
+)
+
+__version__ = "0.1.0"

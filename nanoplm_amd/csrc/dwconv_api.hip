@@ -1,0 +1,375 @@
+// C ABI of libnplm_dwconv (see include/nplm_dwconv.h): argument checks, launch planning and
+// dispatch to the per-K launchers. Host code only; the kernels live in dwconv_kernels.h.
+//
+// The entry points stand where a conv module's forward/backward would sit on the reference's
+// packed path (src/nanoplm/pretraining/models/modern_bert/modeling.py:421-439; backward driven by
+// src/nanoplm/pretraining/pure_pipeline.py:739-742). The reference holds no such op to replace.
+#include <hip/hip_runtime.h>
+
+#include <limits.h>
+#include <stdlib.h>
+
+#include <vector>
+
+#include "../../include/nplm_dwconv.h"
+#include "dwconv_internal.h"
+
+namespace nplm {
+namespace {
+
+constexpr int kVersion = 100;   // 0.1.0
+
+// MI355X: 256 CUs in 8 XCDs. Geometry is a pure function of the problem size so that the
+// reduction order (and with it every output bit) is reproducible.
+constexpr int kNumCU = 256;
+constexpr int kNumXCD = 8;
+constexpr long long kMaxRows = (long long)INT_MAX - (1 << 20);   // row arithmetic is int32 with tile-sized slack
+constexpr int kMaxTileRows = 1 << 16;
+constexpr size_t kSlabBudgetBytes = 16u << 20;   // cap on dw/db partials (written once, read once)
+
+bool specialised_k(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 15 || K == 31; }
+
+int pow2_floor(int v) { int p = 1; while (p * 2 <= v) p *= 2; return p; }
+int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
+
+struct Plan {
+    bool generic;
+    int vec, unroll, maxt;
+    int R, ntiles, ncols, nwc, bw, bt, ncb, nbt, remap;
+};
+
+int default_vec(bool bwd, bool bf16, int K) { return max_vec(bwd, bf16, K); }
+
+// Largest VEC <= cap that divides C, keeps every row slice aligned, and still spreads a row over a
+// whole wave (C / VEC >= 64) unless nothing smaller is left.
+int pick_vec(bool bf16, int C, int cap, uintptr_t align_bits) {
+    const int E = bf16 ? 2 : 4;
+    const int vmax = bf16 ? 8 : 4;
+    for (int v = (cap < vmax ? cap : vmax); v > 1; v >>= 1) {
+        if (C % v) continue;
+        if (align_bits % (uintptr_t)(v * E)) continue;
+        if (C / v < 64) continue;
+        return v;
+    }
+    return 1;
+}
+
+// tune may be null. Returns 0 or a negative argument error.
+int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits,
+              const nplm_dwconv_tuning* tune, Plan* out) {
+    Plan p{};
+    nplm_dwconv_tuning z{};
+    if (!tune) tune = &z;
+    p.generic = !specialised_k(K);
+    const int vcap = tune->vec > 0 ? tune->vec : default_vec(bwd, bf16, K);
+    p.vec = p.generic ? 1 : pick_vec(bf16, C, vcap, align_bits);
+    if (tune->vec > 0 && p.vec != tune->vec) return -NPLM_DWCONV_ETUNING;
+    p.unroll = tune->unroll > 0 ? tune->unroll : default_unroll(bwd, K, p.vec);
+    p.maxt = tune->maxt > 0 ? tune->maxt : default_maxt(bwd, K, p.vec);
+    if (p.maxt < 64 || p.maxt > 1024 || p.maxt % 64) return -NPLM_DWCONV_ETUNING;
+    int R = tune->tile_rows > 0 ? tune->tile_rows : 64;
+    if (R > kMaxTileRows || p.unroll > 64) return -NPLM_DWCONV_ETUNING;
+    R = ceil_div(R, p.unroll) * p.unroll;
+    p.R = R;
+    p.ntiles = ceil_div(T, R);
+    p.ncols = C / p.vec;
+    p.nwc = ceil_div(p.ncols, 64);
+    const int wpb_max = p.maxt / 64;
+    p.bt = tune->bt > 0 ? tune->bt : (bwd ? 4 : 2);
+    if (p.bt > wpb_max) p.bt = wpb_max;
+    p.bw = tune->bw > 0 ? tune->bw : pow2_floor(p.nwc);
+    if (p.bw > wpb_max / p.bt) p.bw = wpb_max / p.bt;
+    if (p.bw < 1 || (p.bw & (p.bw - 1))) return -NPLM_DWCONV_ETUNING;
+    p.ncb = ceil_div(p.nwc, p.bw);
+    const int waves_per_cu = 8;
+    int nbt = tune->nbt > 0 ? tune->nbt : (kNumCU * waves_per_cu) / (p.ncb * p.bw * p.bt);
+    const int nbt_useful = ceil_div(p.ntiles, p.bt);
+    if (nbt > nbt_useful) nbt = nbt_useful;
+    if (bwd) {
+        const size_t slab = (size_t)(K + 1) * C * sizeof(float);
+        const long long cap = (long long)(kSlabBudgetBytes / slab);
+        if (tune->nbt <= 0 && nbt > cap) nbt = (int)cap;
+    }
+    if (nbt < 1) nbt = 1;
+    // keep the grid a multiple of the XCD count when it is large enough, so the remap applies
+    if (tune->nbt <= 0 && nbt >= kNumXCD) nbt -= nbt % kNumXCD;
+    p.nbt = nbt;
+    p.remap = (tune->xcd_remap != 2) && ((long long)p.ncb * p.nbt) % kNumXCD == 0;
+    *out = p;
+    return 0;
+}
+
+void fill_args(const Plan& p, ConvArgs* a) {
+    a->R = p.R; a->ntiles = p.ntiles; a->ncols = p.ncols; a->nwc = p.nwc;
+    a->bw = p.bw; a->bt = p.bt; a->ncb = p.ncb; a->nbt = p.nbt; a->xcd_remap = p.remap;
+}
+
+int check_common(long long T, int C, int K, int S, int act_dtype, int w_dtype) {
+    if (T < 0 || T > kMaxRows || C < 1 || S < 0) return -NPLM_DWCONV_ESHAPE;
+    if ((long long)C * K > INT_MAX / 8) return -NPLM_DWCONV_ESHAPE;
+    if (K < 1 || K > NPLM_DWCONV_MAX_K || (K % 2) == 0) return -NPLM_DWCONV_EKSIZE;
+    if ((act_dtype != NPLM_DWCONV_F32 && act_dtype != NPLM_DWCONV_BF16) ||
+        (w_dtype != NPLM_DWCONV_F32 && w_dtype != NPLM_DWCONV_BF16))
+        return -NPLM_DWCONV_EDTYPE;
+    return 0;
+}
+
+hipError_t launch_fwd(int K, bool bf16, const Plan& p, const ConvArgs& a, dim3 grid, dim3 block, hipStream_t s) {
+    switch (K) {
+        case 3: return launch_fwd_k3(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 5: return launch_fwd_k5(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 7: return launch_fwd_k7(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 9: return launch_fwd_k9(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 15: return launch_fwd_k15(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 31: return launch_fwd_k31(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+    }
+    return hipErrorInvalidConfiguration;
+}
+hipError_t launch_bwd(int K, bool bf16, const Plan& p, const ConvArgs& a, dim3 grid, dim3 block, size_t shmem,
+                      hipStream_t s) {
+    switch (K) {
+        case 3: return launch_bwd_k3(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 5: return launch_bwd_k5(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 7: return launch_bwd_k7(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 9: return launch_bwd_k9(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 15: return launch_bwd_k15(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 31: return launch_bwd_k31(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+    }
+    return hipErrorInvalidConfiguration;
+}
+
+__global__ void fill_zero_kernel(float* p, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0.f;
+}
+hipError_t fill_zero(float* p, long long n, hipStream_t s) {
+    if (!p || n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n);
+    return hipGetLastError();
+}
+
+int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T, int32_t C,
+             int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
+             const nplm_dwconv_tuning* tune) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    if (T == 0) return 0;
+    if (!x || !cu || !w || !y) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t E = bf16 ? 2 : 4;
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
+    if (bits % E) return -NPLM_DWCONV_EALIGN;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
+    Plan p;
+    rc = make_plan(false, bf16, T, C, K, bits, tune, &p);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    if (p.generic) {
+        const int wpb = 4;
+        int blocks = ceil_div(T, wpb);
+        if (blocks > kNumCU * 16) blocks = kNumCU * 16;
+        if (bf16)
+            hipLaunchKernelGGL(dwconv_generic_rows_kernel<true>, dim3(blocks), dim3(wpb * 64), 0, s, x, cu, w, b, y,
+                               (int)T, C, S, K, (int)(w_dtype == NPLM_DWCONV_BF16), 0);
+        else
+            hipLaunchKernelGGL(dwconv_generic_rows_kernel<false>, dim3(blocks), dim3(wpb * 64), 0, s, x, cu, w, b, y,
+                               (int)T, C, S, K, (int)(w_dtype == NPLM_DWCONV_BF16), 0);
+        return (int)hipGetLastError();
+    }
+    ConvArgs a{};
+    a.x = x; a.dy = nullptr; a.cu = cu; a.w = w; a.b = b; a.out = y; a.partial = nullptr;
+    a.T = (int32_t)T; a.C = C; a.S = S; a.K = K; a.w_bf16 = (w_dtype == NPLM_DWCONV_BF16);
+    fill_args(p, &a);
+    const hipError_t e = launch_fwd(K, bf16, p, a, dim3(p.ncb * p.nbt), dim3(p.bw * p.bt * 64), s);
+    if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
+    return (int)e;
+}
+
+int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw, float* db,
+             void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K, int32_t S,
+             int32_t act_dtype, int32_t w_dtype, void* stream, const nplm_dwconv_tuning* tune) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    const bool want_red = dw || db;
+    if (T == 0) {
+        hipError_t e = fill_zero(dw, (long long)C * K, s);
+        if (e == hipSuccess) e = fill_zero(db, C, s);
+        return (int)e;
+    }
+    if (!dx && !want_red) return 0;
+    if (!dy || !cu || !w || (want_red && !x)) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t E = bf16 ? 2 : 4;
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx;
+    if (bits % E) return -NPLM_DWCONV_EALIGN;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
+
+    Plan p;
+    rc = make_plan(true, bf16, T, C, K, bits, tune, &p);
+    if (rc) return rc;
+    if (!tune) {
+        // never use more slabs than nplm_dwconv_bwd_workspace_bytes() promised for aligned inputs
+        Plan nominal;
+        rc = make_plan(true, bf16, T, C, K, 0, nullptr, &nominal);
+        if (rc) return rc;
+        if (p.nbt > nominal.nbt) {
+            p.nbt = nominal.nbt;
+            p.remap = p.remap && ((long long)p.ncb * p.nbt) % kNumXCD == 0;
+        }
+    }
+    const size_t slab = (size_t)(K + 1) * C * sizeof(float);
+    float* partial = nullptr;
+    if (want_red) {
+        if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab * (size_t)p.nbt)
+            return -NPLM_DWCONV_EWORKSPACE;
+        partial = reinterpret_cast<float*>(workspace);
+    }
+    const int w_bf16 = (w_dtype == NPLM_DWCONV_BF16);
+
+    if (p.generic) {
+        if (dx) {
+            const int wpb = 4;
+            int blocks = ceil_div(T, wpb);
+            if (blocks > kNumCU * 16) blocks = kNumCU * 16;
+            if (bf16)
+                hipLaunchKernelGGL(dwconv_generic_rows_kernel<true>, dim3(blocks), dim3(wpb * 64), 0, s, dy, cu, w,
+                                   (const void*)nullptr, dx, (int)T, C, S, K, w_bf16, 1);
+            else
+                hipLaunchKernelGGL(dwconv_generic_rows_kernel<false>, dim3(blocks), dim3(wpb * 64), 0, s, dy, cu, w,
+                                   (const void*)nullptr, dx, (int)T, C, S, K, w_bf16, 1);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return (int)e;
+        }
+        if (want_red) {
+            const int rows = ceil_div(T, p.nbt);
+            const dim3 grid(p.nbt, ceil_div(C, 256));
+            if (bf16)
+                hipLaunchKernelGGL(dwconv_generic_dw_kernel<true>, grid, dim3(256), 0, s, x, dy, cu, partial, (int)T, C,
+                                   S, K, rows);
+            else
+                hipLaunchKernelGGL(dwconv_generic_dw_kernel<false>, grid, dim3(256), 0, s, x, dy, cu, partial, (int)T,
+                                   C, S, K, rows);
+            const hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return (int)e;
+        }
+    } else {
+        ConvArgs a{};
+        // dx-only calls never touch x; point it at dy so the loads stay valid
+        a.x = x ? x : dy; a.dy = dy; a.cu = cu; a.w = w; a.b = nullptr; a.out = dx; a.partial = partial;
+        a.T = (int32_t)T; a.C = C; a.S = S; a.K = K; a.w_bf16 = w_bf16;
+        fill_args(p, &a);
+        const size_t shmem = (size_t)p.bw * p.bt * p.vec * 64 * sizeof(float);
+        const hipError_t e = launch_bwd(K, bf16, p, a, dim3(p.ncb * p.nbt), dim3(p.bw * p.bt * 64), shmem, s);
+        if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
+        if (e != hipSuccess) return (int)e;
+    }
+    if (want_red) {
+        const long long n_out = (long long)(K + 1) * C;
+        hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                           (const float*)partial, p.nbt, C, K, dw, db);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+}
+
+}  // namespace
+}  // namespace nplm
+
+using namespace nplm;
+
+extern "C" {
+
+int nplm_dwconv_version(void) { return kVersion; }
+
+const char* nplm_dwconv_strerror(int code) {
+    if (code == 0) return "success";
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    switch (-code) {
+        case NPLM_DWCONV_ENULL: return "nplm_dwconv: a required pointer is NULL";
+        case NPLM_DWCONV_ESHAPE: return "nplm_dwconv: invalid sizes (need 0 <= T <= INT32_MAX, C >= 1, S >= 0)";
+        case NPLM_DWCONV_EKSIZE: return "nplm_dwconv: kernel size must be odd and in [1, 255]";
+        case NPLM_DWCONV_EDTYPE: return "nplm_dwconv: unknown element type (0 = fp32, 1 = bf16)";
+        case NPLM_DWCONV_EALIGN: return "nplm_dwconv: pointer not aligned to its element size";
+        case NPLM_DWCONV_EWORKSPACE: return "nplm_dwconv: workspace NULL, not 256-byte aligned, or too small";
+        case NPLM_DWCONV_ECU: return "nplm_dwconv: cu_seqlens must start at 0, be non-decreasing and end at T";
+        case NPLM_DWCONV_ETUNING: return "nplm_dwconv: geometry override not available in this build";
+    }
+    return "nplm_dwconv: unknown error code";
+}
+
+int nplm_dwconv_fwd(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T, int32_t C,
+                    int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream) {
+    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, stream, nullptr);
+}
+
+int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T,
+                          int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
+                          const nplm_dwconv_tuning* tune) {
+    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, stream, tune);
+}
+
+size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
+    if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    Plan p;
+    if (make_plan(true, act_dtype == NPLM_DWCONV_BF16, T, C, K, 0, nullptr, &p)) return 0;
+    const size_t bytes = (size_t)p.nbt * (K + 1) * C * sizeof(float);
+    return (bytes + 255) & ~(size_t)255;
+}
+
+int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune) {
+    if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    Plan p;
+    if (make_plan(true, act_dtype == NPLM_DWCONV_BF16, T, C, K, 0, tune, &p)) return 0;
+    return p.nbt;
+}
+
+int nplm_dwconv_bwd(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw, float* db,
+                    void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K, int32_t S,
+                    int32_t act_dtype, int32_t w_dtype, void* stream) {
+    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, stream,
+                    nullptr);
+}
+
+int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw,
+                          float* db, void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K,
+                          int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
+                          const nplm_dwconv_tuning* tune) {
+    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, stream,
+                    tune);
+}
+
+int64_t nplm_dwconv_debug_intervals(const int32_t* cu_host, int32_t S, int64_t T, int64_t start, int64_t step,
+                                    int64_t relocate_every, int32_t* cs_out, int32_t* ce_out) {
+    if (!cu_host || !cs_out || !ce_out || S < 0 || T < 0 || T > kMaxRows || start < 0 || step < 1) return -1;
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    int64_t n = 0;
+    for (int64_t t = start; t < T; t += step, ++n) {
+        if (n == 0 || (relocate_every > 0 && n % relocate_every == 0))
+            sc.locate(cu_host, S, (int)T, (int)t, sc.seq);
+        else
+            sc.advance(cu_host, S, (int)T, (int)t);
+        cs_out[n] = sc.cs;
+        ce_out[n] = sc.ce;
+    }
+    return n;
+}
+
+int nplm_dwconv_check_cu(const int32_t* cu, int32_t S, int64_t T, void* stream) {
+    if (!cu) return -NPLM_DWCONV_ENULL;
+    if (S < 0 || T < 0 || T > kMaxRows) return -NPLM_DWCONV_ESHAPE;
+    std::vector<int32_t> h((size_t)S + 1);
+    hipError_t e = hipMemcpyAsync(h.data(), cu, h.size() * sizeof(int32_t), hipMemcpyDeviceToHost, (hipStream_t)stream);
+    if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+    if (e != hipSuccess) return (int)e;
+    if (h[0] != 0 || h[S] != (int32_t)T) return -NPLM_DWCONV_ECU;
+    for (int32_t i = 0; i < S; ++i)
+        if (h[i + 1] < h[i]) return -NPLM_DWCONV_ECU;
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,135 @@
+// Device-side building blocks of the varlen depthwise conv kernels (gfx950, wave64).
+//
+//  - RowVec<BF16, VEC>: one lane's slice of a token row (VEC adjacent channels) in its memory
+//    format, with the widest load/store the slice allows (16 B for 8 bf16 / 4 fp32).
+//  - SeqCursor: wave-uniform cursor over cu_seqlens; tells which [cs, ce) interval a row is in.
+//
+// The reference (peymanvahidi/nanoplm 0.1.6) has no counterpart: its packed path carries
+// (total_tokens, hidden) activations and int32 cu_seqlens
+// (src/nanoplm/pretraining/models/modern_bert/modeling.py:339, collator.py:322-325), which is the
+// layout these helpers address.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace nplm {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+
+// Two fp32 -> packed bf16 pair, round-to-nearest-even (one v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    f32x2 v = {lo, hi};
+    bf16x2 r = __builtin_convertvector(v, bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    __bf16 r = (__bf16)f;
+    return __builtin_bit_cast(uint16_t, r);
+}
+
+// ---------------------------------------------------------------------------------------------
+// RowVec: VEC adjacent channels of one row, as stored in memory.
+// ---------------------------------------------------------------------------------------------
+template <bool BF16, int VEC> struct RowVec;
+
+// bf16, VEC even: VEC/2 dwords
+template <int VEC> struct RowVec<true, VEC> {
+    static_assert(VEC == 2 || VEC == 4 || VEC == 8, "bf16 VEC");
+    static constexpr int NDW = VEC / 2;
+    static constexpr int BYTES = VEC * 2;
+    uint32_t d[NDW];
+    __device__ __forceinline__ void load(const char* p) {
+        if constexpr (NDW == 4) { uint4 t = *reinterpret_cast<const uint4*>(p); d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w; }
+        else if constexpr (NDW == 2) { uint2 t = *reinterpret_cast<const uint2*>(p); d[0] = t.x; d[1] = t.y; }
+        else { d[0] = *reinterpret_cast<const uint32_t*>(p); }
+    }
+    __device__ __forceinline__ void store(char* p) const {
+        if constexpr (NDW == 4) { *reinterpret_cast<uint4*>(p) = make_uint4(d[0], d[1], d[2], d[3]); }
+        else if constexpr (NDW == 2) { *reinterpret_cast<uint2*>(p) = make_uint2(d[0], d[1]); }
+        else { *reinterpret_cast<uint32_t*>(p) = d[0]; }
+    }
+    __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
+#pragma unroll
+        for (int i = 0; i < NDW; ++i) { f[2 * i] = bf16_lo(d[i]); f[2 * i + 1] = bf16_hi(d[i]); }
+    }
+    __device__ __forceinline__ void from_f32(const float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < NDW; ++i) d[i] = pack_bf16x2(f[2 * i], f[2 * i + 1]);
+    }
+};
+template <> struct RowVec<true, 1> {
+    static constexpr int BYTES = 2;
+    uint16_t h;
+    __device__ __forceinline__ void load(const char* p) { h = *reinterpret_cast<const uint16_t*>(p); }
+    __device__ __forceinline__ void store(char* p) const { *reinterpret_cast<uint16_t*>(p) = h; }
+    __device__ __forceinline__ void to_f32(float (&f)[1]) const { f[0] = bf16_to_f32(h); }
+    __device__ __forceinline__ void from_f32(const float (&f)[1]) { h = f32_to_bf16(f[0]); }
+};
+// fp32
+template <int VEC> struct RowVec<false, VEC> {
+    static_assert(VEC == 1 || VEC == 2 || VEC == 4, "fp32 VEC");
+    static constexpr int BYTES = VEC * 4;
+    float v[VEC];
+    __device__ __forceinline__ void load(const char* p) {
+        if constexpr (VEC == 4) { float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+        else if constexpr (VEC == 2) { float2 t = *reinterpret_cast<const float2*>(p); v[0] = t.x; v[1] = t.y; }
+        else { v[0] = *reinterpret_cast<const float*>(p); }
+    }
+    __device__ __forceinline__ void store(char* p) const {
+        if constexpr (VEC == 4) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+        else if constexpr (VEC == 2) { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
+        else { *reinterpret_cast<float*>(p) = v[0]; }
+    }
+    __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) f[i] = v[i];
+    }
+    __device__ __forceinline__ void from_f32(const float (&f)[VEC]) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) v[i] = f[i];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// SeqCursor: which sequence interval [cs, ce) holds row t. Every member is wave-uniform (the
+// callers derive t from blockIdx and a readfirstlane'd wave index), so the compiler keeps the
+// cursor in scalar registers and reads cu through the scalar (read-only) data path.
+//
+// cu is used ONLY to mask taps, never to form an address, so a malformed cu cannot make the
+// kernels read or write out of bounds. Rows below cu[0] or at/after cu[S] fall into one extra
+// pseudo-sequence on that side.
+// ---------------------------------------------------------------------------------------------
+struct SeqCursor {
+    int seq;  // index of the current interval; -1 / S for the pseudo-sequences at either end
+    int cs;   // first row of the interval
+    int ce;   // one past the last row
+
+    // Position on the interval containing row t, searching cu[hint..S].
+    __host__ __device__ __forceinline__ void locate(const int32_t* __restrict__ cu, int S, int T, int t, int hint) {
+        int lo = hint < 0 ? 0 : hint, hi = S;
+        // first i in [lo, S) with cu[i+1] > t, else S
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (cu[mid + 1] > t) hi = mid; else lo = mid + 1;
+        }
+        seq = lo;
+        if (lo < S) { cs = cu[lo]; ce = cu[lo + 1]; }
+        else        { cs = cu[S];  ce = T; }
+        if (cs > t) { ce = cs; cs = 0; seq = -1; }   // row lies before cu[0]
+    }
+    // Move forward until the interval contains row t (t must not decrease between calls).
+    __host__ __device__ __forceinline__ void advance(const int32_t* __restrict__ cu, int S, int T, int t) {
+        while (t >= ce && seq < S) {
+            ++seq;
+            cs = ce;
+            ce = (seq < S) ? cu[seq + 1] : T;
+        }
+    }
+};
+
+}  // namespace nplm

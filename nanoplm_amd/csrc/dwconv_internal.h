@@ -1,0 +1,86 @@
+// Host-side internals of libnplm_dwconv: launch plans, the per-K launcher tables, and the
+// geometry-override entry points used by the benchmark sweeps and the geometry tests.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "dwconv_kernels.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// Launch-geometry overrides; a field left 0 keeps the library's default for that field.
+typedef struct nplm_dwconv_tuning {
+    int32_t vec;        // channels per lane (bf16: 1,2,4,8; fp32: 1,2,4)
+    int32_t unroll;     // output rows per chunk (U); must be one the library was built with
+    int32_t tile_rows;  // rows per tile (R), rounded up to a multiple of unroll
+    int32_t bw;         // wave-columns per block (power of two)
+    int32_t bt;         // token slots per block
+    int32_t nbt;        // token-blocks in the grid
+    int32_t xcd_remap;  // 1 = on, 2 = off
+    int32_t maxt;       // launch-bounds class (threads per block the kernel was compiled for)
+} nplm_dwconv_tuning;
+
+// Same contracts as nplm_dwconv_fwd / nplm_dwconv_bwd, with geometry overrides. An override the
+// build does not hold a kernel for yields -NPLM_DWCONV_ETUNING.
+#define NPLM_DWCONV_ETUNING 8
+int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const void* b, void* y,
+                          int64_t T, int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype,
+                          void* stream, const nplm_dwconv_tuning* tune);
+int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx,
+                          float* dw, float* db, void* workspace, size_t workspace_bytes, int64_t T,
+                          int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype,
+                          void* stream, const nplm_dwconv_tuning* tune);
+// Token-blocks (= workspace slabs of (K+1)*C floats) a backward launch with these overrides uses.
+int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune);
+
+// Host-side run of the kernels' boundary cursor (SeqCursor) over a HOST copy of cu: for rows
+// t = start, start+step, ... < T writes the interval [cs, ce) the cursor reports, located afresh
+// at `start` and every `relocate_every` rows (0 = never) and advanced in between -- the same two
+// moves the kernels make at tile starts and inside tiles. Returns the number of rows written.
+int64_t nplm_dwconv_debug_intervals(const int32_t* cu_host, int32_t S, int64_t T, int64_t start, int64_t step,
+                                    int64_t relocate_every, int32_t* cs_out, int32_t* ce_out);
+
+#ifdef __cplusplus
+}
+#endif
+
+namespace nplm {
+
+// One launcher per specialised kernel size, each in its own translation unit.
+// Return hipErrorInvalidConfiguration when the (vec, unroll, maxt) combination is not built.
+#define NPLM_DECLARE_K(KK)                                                                              \
+    hipError_t launch_fwd_k##KK(bool bf16, int vec, int unroll, int maxt, const ConvArgs& a, dim3 grid, \
+                                dim3 block, hipStream_t s);                                             \
+    hipError_t launch_bwd_k##KK(bool bf16, int vec, int unroll, int maxt, const ConvArgs& a, dim3 grid, \
+                                dim3 block, size_t shmem, hipStream_t s);
+NPLM_DECLARE_K(3)
+NPLM_DECLARE_K(5)
+NPLM_DECLARE_K(7)
+NPLM_DECLARE_K(9)
+NPLM_DECLARE_K(15)
+NPLM_DECLARE_K(31)
+#undef NPLM_DECLARE_K
+
+// Widest lane slice (channels per lane) built for a (pass, dtype, K), default chunk length U and
+// launch-bounds class for a (pass, K, VEC) — the single place both the instantiation lists and the
+// planner read. Wider slices than these spill registers.
+constexpr int max_vec(bool bwd, bool bf16, int K) {
+    if (!bf16) return K >= 15 ? 1 : (bwd ? 2 : 4);
+    if (K >= 31) return bwd ? 1 : 2;
+    if (K >= 15) return bwd ? 2 : 4;
+    return bwd ? 4 : 8;
+}
+constexpr int default_unroll(bool bwd, int K, int vec) {
+    (void)bwd;
+    if (K >= 15) return 4;
+    return vec >= 8 ? 4 : 8;
+}
+constexpr int default_maxt(bool bwd, int K, int vec) {
+    (void)K; (void)vec;
+    return bwd ? 512 : 256;
+}
+
+}  // namespace nplm

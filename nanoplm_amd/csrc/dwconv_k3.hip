@@ -1,0 +1,3 @@
+// Sliding-window forward / fused backward kernels specialised for kernel size 3.
+#define NPLM_K 3
+#include "dwconv_inst.inc"

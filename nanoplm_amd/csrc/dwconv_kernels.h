@@ -1,0 +1,495 @@
+// Kernels of the varlen depthwise conv (gfx950, wave64): sliding-window forward, fused backward
+// (dx + dw/db partials), partial-sum finalize, and runtime-K fallbacks.
+//
+// Work decomposition (forward and backward share it)
+// --------------------------------------------------
+//   thread-column : VEC adjacent channels, one lane; ncols = C / VEC
+//   wave-column   : 64 adjacent thread-columns (64*VEC channels); nwc = ceil(ncols / 64)
+//   tile          : R consecutive token rows; ntiles = ceil(T / R)
+//   wave-item     : (tile, wave-column). A wave walks its tile top to bottom, holding the last
+//                   K-1 rows in registers as fp32, so inside a tile every row is loaded once;
+//                   only the K-1 rows around a tile edge are loaded by both neighbours.
+//   block         : bw wave-columns x bt token slots (bw*bt waves).
+//   grid          : ncb column-blocks x nbt token-blocks. Token slot s = tb*bt + tl walks tiles
+//                   s, s + ntslots, s + 2*ntslots, ... (ntslots = nbt*bt), so at any moment the
+//                   resident waves cover one contiguous window of rows that sweeps through the
+//                   tensor, and the backward accumulates dw/db in registers over all its tiles.
+//
+// Sequence boundaries: the wave keeps a scalar cursor over cu (SeqCursor). A chunk of U output
+// rows whose whole footprint [t-P, t+U-1+P] lies inside one sequence takes the unmasked path;
+// otherwise every tap is selected (not multiplied) against [cs, ce) of its output row, so values
+// from another sequence, NaN/Inf included, never enter a sum.
+//
+// No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); the tensor
+// contract is the packed path's: modeling.py:339,421-439 and collator.py:322-325,405-458.
+#pragma once
+#include "dwconv_device.h"
+
+namespace nplm {
+
+struct ConvArgs {
+    const void* x;         // fwd: x          bwd: x
+    const void* dy;        // fwd: unused     bwd: dy
+    const int32_t* cu;     // [S+1]
+    const void* w;         // [C,K] f32 or bf16
+    const void* b;         // fwd: [C] or null
+    void* out;             // fwd: y          bwd: dx (may be null)
+    float* partial;        // bwd: [nbt][K+1][C] fp32 (may be null -> no dw/db)
+    int32_t T, C, S, K;
+    int32_t w_bf16;
+    // geometry
+    int32_t R;             // rows per tile (multiple of U)
+    int32_t ntiles;        // ceil(T / R)
+    int32_t ncols;         // C / VEC
+    int32_t nwc;           // ceil(ncols / 64)
+    int32_t bw, bt;        // block = bw wave-columns x bt token slots
+    int32_t ncb, nbt;      // grid = ncb x nbt blocks
+    int32_t xcd_remap;     // 1: blocks that share an XCD get adjacent token-blocks (needs nblocks % 8 == 0)
+};
+
+__device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+// blockIdx -> (column-block, token-block). Hardware deals consecutive workgroups round-robin to the
+// 8 XCDs; with xcd_remap, workgroups on one XCD get consecutive logical ids, so tiles that share
+// halo rows meet in the same L2.
+__device__ __forceinline__ void block_coords(const ConvArgs& a, int& cb, int& tb) {
+    int b = (int)blockIdx.x;
+    if (a.xcd_remap) {
+        const int per = (int)(gridDim.x >> 3);
+        b = (b & 7) * per + (b >> 3);
+    }
+    cb = b % a.ncb;
+    tb = b / a.ncb;
+}
+
+template <int VEC, int K>
+__device__ __forceinline__ void load_weights(const ConvArgs& a, int c0, float (&wr)[VEC][K]) {
+    if (a.w_bf16) {
+        const uint16_t* wp = reinterpret_cast<const uint16_t*>(a.w) + (size_t)c0 * K;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+#pragma unroll
+            for (int k = 0; k < K; ++k) wr[v][k] = bf16_to_f32(wp[v * K + k]);
+    } else {
+        const float* wp = reinterpret_cast<const float*>(a.w) + (size_t)c0 * K;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+#pragma unroll
+            for (int k = 0; k < K; ++k) wr[v][k] = wp[v * K + k];
+    }
+}
+
+__device__ __forceinline__ int clamp_row(int r, int T) { return r < 0 ? 0 : (r >= T ? T - 1 : r); }
+
+// =============================================================================================
+// Forward
+// =============================================================================================
+template <bool BF16, int K, int VEC, int U, int MAXT>
+__global__ void __launch_bounds__(MAXT) dwconv_fwd_kernel(const ConvArgs a) {
+    constexpr int P = (K - 1) / 2;
+    constexpr int E = BF16 ? 2 : 4;
+    using Row = RowVec<BF16, VEC>;
+
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    int cb, tb;
+    block_coords(a, cb, tb);
+    const int wc = cb * a.bw + (wv % a.bw);
+    const int tslot = tb * a.bt + (wv / a.bw);
+    const int ntslots = a.nbt * a.bt;
+    if (wc >= a.nwc) return;
+
+    const int col = wc * 64 + lane;
+    const bool active = col < a.ncols;
+    const int c0 = (active ? col : a.ncols - 1) * VEC;   // clamped: loads stay in bounds, stores are guarded
+    const uint32_t lane_off = (uint32_t)c0 * E;
+    const size_t row_bytes = (size_t)a.C * E;
+    const int T = a.T, S = a.S, R = a.R;
+    const int32_t* __restrict__ cu = a.cu;
+    const char* __restrict__ xb = reinterpret_cast<const char*>(a.x);
+    char* __restrict__ yb = reinterpret_cast<char*>(a.out);
+
+    float wr[VEC][K];
+    load_weights<VEC, K>(a, c0, wr);
+    float bias[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
+    if (a.b) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+            bias[v] = a.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.b)[c0 + v])
+                               : reinterpret_cast<const float*>(a.b)[c0 + v];
+    }
+
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+
+    for (int tile = tslot; tile < a.ntiles; tile += ntslots) {
+        const int t0 = tile * R;
+        const int t1 = (t0 + R < T) ? t0 + R : T;
+        sc.locate(cu, S, T, t0, sc.seq);
+
+        float win[K - 1 + U][VEC];   // win[j] = row (tc - P + j)
+#pragma unroll
+        for (int j = 0; j < K - 1; ++j) {
+            Row r;
+            r.load(xb + (size_t)clamp_row(t0 - P + j, T) * row_bytes + lane_off);
+            r.to_f32(win[j]);
+        }
+        Row nxt[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) nxt[u].load(xb + (size_t)clamp_row(t0 + P + u, T) * row_bytes + lane_off);
+
+        for (int tc = t0; tc < t1; tc += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) nxt[u].to_f32(win[K - 1 + u]);
+            if (tc + U < t1) {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    nxt[u].load(xb + (size_t)clamp_row(tc + U + P + u, T) * row_bytes + lane_off);
+            }
+            sc.advance(cu, S, T, tc);
+            if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
+                // whole footprint inside one sequence
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    float acc[VEC];
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+#pragma unroll
+                    for (int k = 0; k < K; ++k)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wr[v][k], win[u + k][v], acc[v]);
+                    Row o;
+                    o.from_f32(acc);
+                    if (active) o.store(yb + (size_t)(tc + u) * row_bytes + lane_off);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int t = tc + u;
+                    if (t < t1) {
+                        sc.advance(cu, S, T, t);
+                        float acc[VEC];
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+#pragma unroll
+                        for (int k = 0; k < K; ++k) {
+                            const int j = t + k - P;
+                            const bool ok = (j >= sc.cs) && (j < sc.ce);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) {
+                                const float xv = ok ? win[u + k][v] : 0.f;
+                                acc[v] = __builtin_fmaf(wr[v][k], xv, acc[v]);
+                            }
+                        }
+                        Row o;
+                        o.from_f32(acc);
+                        if (active) o.store(yb + (size_t)t * row_bytes + lane_off);
+                    }
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) win[j][v] = win[j + U][v];
+        }
+    }
+}
+
+// =============================================================================================
+// Backward (fused): dx, plus per-block partial sums of dw and db
+// =============================================================================================
+// Row t contributes   dx[t]   = sum_m w[K-1-m] * dy[t-P+m]   (m over the window, masked)
+//                     dw[k]  += dy[t] * x[t-P+k]             (masked the same way)
+//                     db     += dy[t]
+// Each wave keeps dw/db for its VEC channels in registers across all its tiles. At the end the bt
+// waves of a block that share a wave-column are summed through LDS in fixed order (token slot
+// 0,1,2,...), and the block writes one slab partial[tb][k][c]. No atomics.
+template <bool BF16, int K, int VEC, int U, int MAXT>
+__global__ void __launch_bounds__(MAXT) dwconv_bwd_kernel(const ConvArgs a) {
+    constexpr int P = (K - 1) / 2;
+    constexpr int E = BF16 ? 2 : 4;
+    using Row = RowVec<BF16, VEC>;
+    extern __shared__ float red[];   // [nwaves][VEC][64]
+
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    int cb, tb;
+    block_coords(a, cb, tb);
+    const int wcl = wv % a.bw;
+    const int tl = wv / a.bw;
+    const int wc = cb * a.bw + wcl;
+    const int tslot = tb * a.bt + tl;
+    const int ntslots = a.nbt * a.bt;
+    const bool wave_on = wc < a.nwc;   // idle waves still take part in the barriers below
+
+    const int col = wc * 64 + lane;
+    const bool active = wave_on && col < a.ncols;
+    const int c0 = (active ? col : a.ncols - 1) * VEC;
+    const uint32_t lane_off = (uint32_t)c0 * E;
+    const size_t row_bytes = (size_t)a.C * E;
+    const int T = a.T, S = a.S, R = a.R;
+    const int32_t* __restrict__ cu = a.cu;
+    const char* __restrict__ xb = reinterpret_cast<const char*>(a.x);
+    const char* __restrict__ gb = reinterpret_cast<const char*>(a.dy);
+    char* __restrict__ ob = reinterpret_cast<char*>(a.out);
+    const bool want_dx = ob != nullptr;
+    const bool want_dw = a.partial != nullptr;
+
+    float wr[VEC][K];
+    load_weights<VEC, K>(a, c0, wr);
+    float dwa[VEC][K];
+    float dba[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        dba[v] = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) dwa[v][k] = 0.f;
+    }
+
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+
+    if (wave_on) {
+        for (int tile = tslot; tile < a.ntiles; tile += ntslots) {
+            const int t0 = tile * R;
+            const int t1 = (t0 + R < T) ? t0 + R : T;
+            sc.locate(cu, S, T, t0, sc.seq);
+
+            float xw[K - 1 + U][VEC];   // x  rows tc-P .. tc+U-1+P
+            float gw[K - 1 + U][VEC];   // dy rows, same range
+#pragma unroll
+            for (int j = 0; j < K - 1; ++j) {
+                const size_t off = (size_t)clamp_row(t0 - P + j, T) * row_bytes + lane_off;
+                Row r;
+                r.load(xb + off); r.to_f32(xw[j]);
+                r.load(gb + off); r.to_f32(gw[j]);
+            }
+            Row nx[U], ng[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const size_t off = (size_t)clamp_row(t0 + P + u, T) * row_bytes + lane_off;
+                nx[u].load(xb + off);
+                ng[u].load(gb + off);
+            }
+
+            for (int tc = t0; tc < t1; tc += U) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) { nx[u].to_f32(xw[K - 1 + u]); ng[u].to_f32(gw[K - 1 + u]); }
+                if (tc + U < t1) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const size_t off = (size_t)clamp_row(tc + U + P + u, T) * row_bytes + lane_off;
+                        nx[u].load(xb + off);
+                        ng[u].load(gb + off);
+                    }
+                }
+                sc.advance(cu, S, T, tc);
+                if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        float g[VEC];
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) { g[v] = gw[u + P][v]; dba[v] += g[v]; }
+#pragma unroll
+                        for (int k = 0; k < K; ++k)
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) dwa[v][k] = __builtin_fmaf(g[v], xw[u + k][v], dwa[v][k]);
+                        if (want_dx) {
+                            float acc[VEC];
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+#pragma unroll
+                            for (int m = 0; m < K; ++m)
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gw[u + m][v], acc[v]);
+                            Row o;
+                            o.from_f32(acc);
+                            if (active) o.store(ob + (size_t)(tc + u) * row_bytes + lane_off);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) {
+                        const int t = tc + u;
+                        if (t < t1) {
+                            sc.advance(cu, S, T, t);
+                            float g[VEC], acc[VEC];
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) { g[v] = gw[u + P][v]; dba[v] += g[v]; acc[v] = 0.f; }
+#pragma unroll
+                            for (int m = 0; m < K; ++m) {
+                                const int j = t + m - P;
+                                const bool ok = (j >= sc.cs) && (j < sc.ce);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    const float xv = ok ? xw[u + m][v] : 0.f;
+                                    const float gv = ok ? gw[u + m][v] : 0.f;
+                                    dwa[v][m] = __builtin_fmaf(g[v], xv, dwa[v][m]);
+                                    acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
+                                }
+                            }
+                            if (want_dx) {
+                                Row o;
+                                o.from_f32(acc);
+                                if (active) o.store(ob + (size_t)t * row_bytes + lane_off);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) { xw[j][v] = xw[j + U][v]; gw[j][v] = gw[j + U][v]; }
+            }
+        }
+    }
+
+    if (!want_dw) return;   // uniform over the grid
+
+    // ---- block-level pass: sum the bt token slots of each wave-column, slot order 0,1,2,... ----
+    float* slab = a.partial + (size_t)tb * (K + 1) * a.C;
+#pragma unroll
+    for (int kk = 0; kk <= K; ++kk) {
+        float val[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) val[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : dba[v];
+        if (tl > 0) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) red[(wv * VEC + v) * 64 + lane] = val[v];
+        }
+        __syncthreads();
+        if (tl == 0) {
+            for (int j = 1; j < a.bt; ++j) {
+                const int ow = j * a.bw + wcl;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
+            }
+            if (active) {
+                float* dst = slab + (size_t)kk * a.C + c0;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) dst[v] = val[v];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// =============================================================================================
+// Finalize: dw[c][k] = sum_p partial[p][k][c], db[c] = sum_p partial[p][K][c], p in fixed order.
+// Block = 64 outputs (adjacent c) x FIN_SPLIT groups of p; each group sums its contiguous share
+// of p in order, then group 0 adds the group sums in order.
+// =============================================================================================
+constexpr int FIN_SPLIT = 8;
+
+template <int SPLIT>
+__global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
+                                       float* __restrict__ dw, float* __restrict__ db) {
+    __shared__ float red[SPLIT][64];
+    const int lane = (int)(threadIdx.x & 63);
+    const int grp = (int)(threadIdx.x >> 6);
+    const long long n_out = (long long)(K + 1) * C;
+    const long long o = (long long)blockIdx.x * 64 + lane;   // o = kk*C + c
+    const bool on = o < n_out;
+    const int per = (nbt + SPLIT - 1) / SPLIT;
+    const int p0 = grp * per;
+    const int p1 = (p0 + per < nbt) ? p0 + per : nbt;
+    float s = 0.f;
+    if (on) {
+        const float* src = partial + o;
+        const size_t stride = (size_t)n_out;
+        for (int p = p0; p < p1; ++p) s += src[(size_t)p * stride];
+    }
+    red[grp][lane] = s;
+    __syncthreads();
+    if (grp == 0 && on) {
+        float tot = red[0][lane];
+#pragma unroll
+        for (int g = 1; g < SPLIT; ++g) tot += red[g][lane];
+        const int kk = (int)(o / C);
+        const int c = (int)(o - (long long)kk * C);
+        if (kk < K) { if (dw) dw[(size_t)c * K + kk] = tot; }
+        else        { if (db) db[c] = tot; }
+    }
+}
+
+// =============================================================================================
+// Runtime-K fallbacks (any odd K, any C): correct, not tuned. One wave per token row, lanes stride
+// over channels.
+// =============================================================================================
+template <bool BF16>
+__device__ __forceinline__ float ld_act(const void* p, size_t i) {
+    if constexpr (BF16) return bf16_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+    else return reinterpret_cast<const float*>(p)[i];
+}
+template <bool BF16>
+__device__ __forceinline__ void st_act(void* p, size_t i, float f) {
+    if constexpr (BF16) reinterpret_cast<uint16_t*>(p)[i] = f32_to_bf16(f);
+    else reinterpret_cast<float*>(p)[i] = f;
+}
+__device__ __forceinline__ float ld_w(const void* p, int w_bf16, size_t i) {
+    return w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p)[i]) : reinterpret_cast<const float*>(p)[i];
+}
+
+// flip = 0: out[t] = b + sum_k w[k] * in[t+k-P]   (forward)
+// flip = 1: out[t] =     sum_k w[k] * in[t-k+P]   (dx from dy)
+template <bool BF16>
+__global__ void dwconv_generic_rows_kernel(const void* in, const int32_t* __restrict__ cu, const void* w,
+                                           const void* b, void* out, int T, int C, int S, int K,
+                                           int w_bf16, int flip) {
+    const int P = (K - 1) / 2;
+    const int lane = (int)(threadIdx.x & 63);
+    const int wpb = (int)(blockDim.x >> 6);
+    const int gw = (int)blockIdx.x * wpb + wave_id();
+    const int nw = (int)gridDim.x * wpb;
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    for (int t = gw; t < T; t += nw) {
+        sc.locate(cu, S, T, t, sc.seq);
+        for (int c = lane; c < C; c += 64) {
+            float acc = (b && !flip) ? ld_w(b, w_bf16, c) : 0.f;
+            for (int k = 0; k < K; ++k) {
+                const int j = flip ? (t - k + P) : (t + k - P);
+                // cu only masks; the explicit [0, T) test keeps a malformed cu from forming a bad address
+                if (j >= sc.cs && j < sc.ce && j >= 0 && j < T)
+                    acc = __builtin_fmaf(ld_w(w, w_bf16, (size_t)c * K + k), ld_act<BF16>(in, (size_t)j * C + c), acc);
+            }
+            st_act<BF16>(out, (size_t)t * C + c, acc);
+        }
+    }
+}
+
+// partial[tb][kk][c] over the rows of token-block tb. grid = (nbt, ceil(C/256)); thread = channel.
+template <bool BF16>
+__global__ void dwconv_generic_dw_kernel(const void* x, const void* dy, const int32_t* __restrict__ cu,
+                                         float* __restrict__ partial, int T, int C, int S, int K, int rows_per_block) {
+    const int P = (K - 1) / 2;
+    const int c = (int)(blockIdx.y * blockDim.x + threadIdx.x);
+    const int tb = (int)blockIdx.x;
+    const long long r0 = (long long)tb * rows_per_block;
+    const int t0 = (int)(r0 < T ? r0 : T);
+    const int t1 = (int)((r0 + rows_per_block < T) ? r0 + rows_per_block : T);
+    float* slab = partial + (size_t)tb * (K + 1) * C;
+    for (int kk = 0; kk <= K; ++kk) {
+        float acc = 0.f;
+        SeqCursor sc;
+        sc.seq = 0; sc.cs = 0; sc.ce = 0;
+        if (t0 < t1) sc.locate(cu, S, T, t0, 0);
+        for (int t = t0; t < t1; ++t) {
+            sc.advance(cu, S, T, t);
+            if (c < C) {
+                const float g = ld_act<BF16>(dy, (size_t)t * C + c);
+                if (kk == K) acc += g;
+                else {
+                    const int j = t + kk - P;
+                    if (j >= sc.cs && j < sc.ce && j >= 0 && j < T)
+                        acc = __builtin_fmaf(g, ld_act<BF16>(x, (size_t)j * C + c), acc);
+                }
+            }
+        }
+        if (c < C) slab[(size_t)kk * C + c] = acc;
+    }
+}
+
+}  // namespace nplm

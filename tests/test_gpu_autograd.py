@@ -1,0 +1,89 @@
+"""GPU tests of the autograd Function / nn.Module surface against the reference path on the CPU."""
+import pytest
+import torch
+
+import nanoplm_amd as npa
+from nanoplm_amd.workloads import make_workload
+from oracle import dwconv_ref as O
+
+from gpu_util import assert_act_close, assert_red_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def test_function_backward_matches_reference_autograd_fp32():
+    wl = make_workload(1, with_dy=True)
+    y_r, dx_r, dw_r, db_r = O.ref_dwconv_varlen_grads(wl.x, wl.cu_seqlens, wl.weight, wl.bias, wl.dy, torch.float64)
+    x = wl.x.to(DEV).requires_grad_(True)
+    w = wl.weight.to(DEV).requires_grad_(True)
+    b = wl.bias.to(DEV).requires_grad_(True)
+    y = npa.VarlenDWConv1dFunction.apply(x, wl.cu_seqlens.to(DEV), w, b)
+    y.backward(wl.dy.to(DEV))
+    assert_act_close(y, y_r, torch.float32, "y")
+    assert_act_close(x.grad, dx_r, torch.float32, "dx")
+    assert_red_close(w.grad, dw_r, "dw")
+    assert_red_close(b.grad, db_r, "db")
+
+
+def test_module_under_autocast_with_fp32_parameters():
+    """bf16 activations with fp32 master parameters, as under torch.autocast in the training loop
+    (src/nanoplm/pretraining/pure_pipeline.py:717-722); gradients come back in the parameters' dtype."""
+    wl = make_workload(5, T=5000, C=512)
+    conv = npa.VarlenDWConv1d(512, 7).to(DEV)
+    with torch.no_grad():
+        conv.weight.copy_(wl.weight.float())
+        conv.bias.copy_(wl.bias.float())
+    x = wl.x.to(DEV).requires_grad_(True)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        y = conv(x, wl.cu_seqlens.to(DEV))
+    assert y.dtype == torch.bfloat16
+    y.backward(wl.dy.to(DEV))
+    assert conv.weight.grad.dtype == torch.float32 and x.grad.dtype == torch.bfloat16
+    y_r, dx_r, dw_r, db_r = O.ref_dwconv_varlen_grads(wl.x, wl.cu_seqlens, wl.weight, wl.bias, wl.dy, torch.float64)
+    assert_act_close(y, y_r, torch.bfloat16, "y")
+    assert_act_close(x.grad, dx_r, torch.bfloat16, "dx")
+    assert_red_close(conv.weight.grad, dw_r, "dw")
+    assert_red_close(conv.bias.grad, db_r, "db")
+
+
+def test_bf16_parameters_get_bf16_gradients_and_frozen_inputs_get_none():
+    wl = make_workload(5, T=3000, C=256)
+    x = wl.x.to(DEV)                                   # no grad wanted for x
+    w = wl.weight.to(DEV).requires_grad_(True)
+    b = wl.bias.to(DEV).requires_grad_(True)
+    y = npa.varlen_dwconv(x, wl.cu_seqlens.to(DEV), w, b)
+    y.backward(wl.dy.to(DEV))
+    assert w.grad.dtype == torch.bfloat16 and b.grad.dtype == torch.bfloat16
+    _, _, dw_r, db_r = O.ref_dwconv_varlen_grads(wl.x, wl.cu_seqlens, wl.weight, wl.bias, wl.dy, torch.float64)
+    # one bf16 rounding of the fp32 result
+    assert bool(((w.grad.double().cpu() - dw_r).abs() <= dw_r.abs() * 2.0 ** -8 + 1e-3).all())
+    assert bool(((b.grad.double().cpu() - db_r).abs() <= db_r.abs() * 2.0 ** -8 + 1e-3).all())
+    # only dx requested
+    x2 = wl.x.to(DEV).requires_grad_(True)
+    y2 = npa.varlen_dwconv(x2, wl.cu_seqlens.to(DEV), w.detach(), b.detach())
+    y2.backward(wl.dy.to(DEV))
+    assert x2.grad is not None
+
+
+def test_non_contiguous_inputs_are_accepted():
+    wl = make_workload(5, T=2000, C=256)
+    xt = wl.x.to(DEV).t().contiguous().t()             # [T, C] view with transposed strides
+    assert not xt.is_contiguous()
+    y = npa.varlen_dwconv_fwd(xt, wl.cu_seqlens.to(DEV), wl.weight.to(DEV), wl.bias.to(DEV))
+    y0 = npa.varlen_dwconv_fwd(wl.x.to(DEV), wl.cu_seqlens.to(DEV), wl.weight.to(DEV), wl.bias.to(DEV))
+    assert torch.equal(y, y0)
+
+
+def test_runs_on_a_side_stream():
+    wl = make_workload(5, T=4000, C=256).to(DEV)
+    y0 = npa.varlen_dwconv_fwd(wl.x, wl.cu_seqlens, wl.weight, wl.bias)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        y1 = npa.varlen_dwconv_fwd(wl.x, wl.cu_seqlens, wl.weight, wl.bias)
+        dx1, dw1, db1 = npa.varlen_dwconv_bwd(wl.x, wl.dy, wl.cu_seqlens, wl.weight)
+    s.synchronize()
+    dx0, dw0, db0 = npa.varlen_dwconv_bwd(wl.x, wl.dy, wl.cu_seqlens, wl.weight)
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1) and torch.equal(db0, db1)

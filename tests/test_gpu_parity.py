@@ -1,0 +1,285 @@
+"""GPU parity of the HIP kernels (called through the C ABI) against the CPU oracle.
+
+Every test here needs a real MI355X. Inputs are the seeded configurations of
+nanoplm_amd.workloads at their full sizes, the committed golden vectors, and edge cases; the oracle
+is oracle/ (C restatement with double accumulation, pinned by tests/test_oracle.py).
+"""
+import numpy as np
+import pytest
+import torch
+
+import nanoplm_amd as npa
+from nanoplm_amd import _lib
+from nanoplm_amd.workloads import cu_from_lengths, make_workload, static_packed_cu
+from oracle import dwconv_ref as O
+
+from gpu_util import assert_act_close, assert_red_close, workload_with_oracle
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _run_all(wl_dev):
+    y = npa.varlen_dwconv_fwd(wl_dev.x, wl_dev.cu_seqlens, wl_dev.weight, wl_dev.bias)
+    dx, dw, db = npa.varlen_dwconv_bwd(wl_dev.x, wl_dev.dy, wl_dev.cu_seqlens, wl_dev.weight)
+    torch.cuda.synchronize()
+    return y, dx, dw, db
+
+
+def test_library_is_loaded_from_the_tree():
+    lib = _lib.load()
+    assert lib.nplm_dwconv_version() >= 100
+    assert torch.cuda.is_available() and "gfx950" in torch.cuda.get_device_properties(0).gcnArchName
+
+
+# ---- the five configurations at full size ---------------------------------------------------------
+@pytest.mark.parametrize("index", [1, 2, 3, 5, 4])
+def test_configuration_matches_oracle(index):
+    print(f"[case] configuration {index}", flush=True)
+    wl, y64, dx64, dw64, db64 = workload_with_oracle(index)
+    d = wl.to(DEV)
+    y, dx, dw, db = _run_all(d)
+    e_y = assert_act_close(y, y64, wl.dtype, f"cfg{index} y")
+    e_dx = assert_act_close(dx, dx64, wl.dtype, f"cfg{index} dx")
+    e_dw = assert_red_close(dw, dw64, f"cfg{index} dw")
+    e_db = assert_red_close(db, db64, f"cfg{index} db")
+    print(f"[parity] cfg{index} T={wl.T} C={wl.C} K={wl.K} S={wl.S} {wl.dtype}: max-abs y {e_y:.3e} dx {e_dx:.3e} "
+          f"dw {e_dw:.3e} (max|dw| {float(dw64.abs().max()):.1f}) db {e_db:.3e}", flush=True)
+    # run-to-run determinism: bit-identical outputs, reductions included
+    y2, dx2, dw2, db2 = _run_all(d)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.equal(db, db2)
+
+
+def test_configuration_1_against_the_fp32_reference_path():
+    """Configuration 1 is defined against the fp32 per-sequence conv1d path itself."""
+    wl = make_workload(1)
+    y_ref = O.ref_dwconv_varlen(wl.x, wl.cu_seqlens, wl.weight, wl.bias, torch.float32)
+    d = wl.to(DEV)
+    y = npa.varlen_dwconv_fwd(d.x, d.cu_seqlens, d.weight, d.bias).cpu()
+    rel = float((y - y_ref).abs().max() / y_ref.abs().max())
+    assert rel <= 1e-5, rel
+
+
+# ---- golden vectors -------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["cfg1_fp32_C64_K3", "boundary_fp32_C16_K7", "stress_bf16_C32_K7"])
+def test_golden_vectors(name, golden_dir):
+    z = np.load(f"{golden_dir}/{name}.npz", allow_pickle=False)
+    dt = torch.bfloat16 if str(z["act_dtype"]) == "bfloat16" else torch.float32
+    x, w, b, dy = (torch.from_numpy(z[k]).to(dt).to(DEV) for k in ("x", "w", "b", "dy"))
+    cu = torch.from_numpy(z["cu_seqlens"]).to(DEV)
+    y = npa.varlen_dwconv_fwd(x, cu, w, b)
+    dx, dw, db = npa.varlen_dwconv_bwd(x, dy, cu, w)
+    assert_act_close(y, torch.from_numpy(z["y"]).double(), dt, name + " y")
+    assert_act_close(dx, torch.from_numpy(z["dx"]).double(), dt, name + " dx")
+    assert_red_close(dw, torch.from_numpy(z["dw"]), name + " dw")
+    assert_red_close(db, torch.from_numpy(z["db"]), name + " db")
+
+
+# ---- shapes, kernel sizes, dtypes -------------------------------------------------------------------
+def _random_case(lens, C, K, dt, wdt, seed=0, bias=True):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.tensor(lens)
+    T = int(lens.sum())
+    x = torch.randn(T, C, generator=g).to(dt)
+    w = (torch.randn(C, K, generator=g) * K ** -0.5).to(wdt)
+    b = (torch.randn(C, generator=g) * 0.02).to(wdt) if bias else None
+    dy = torch.randn(T, C, generator=g).to(dt)
+    return x, cu_from_lengths(lens), w, b, dy
+
+
+def _check_case(x, cu, w, b, dy, what):
+    y64 = O.c_oracle_fwd(x, cu, w, b)
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
+    xd, cud, wd, dyd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV)
+    bd = None if b is None else b.to(DEV)
+    y = npa.varlen_dwconv_fwd(xd, cud, wd, bd)
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    assert_act_close(y, y64, x.dtype, what + " y")
+    assert_act_close(dx, dx64, x.dtype, what + " dx")
+    assert_red_close(dw, dw64, what + " dw")
+    assert_red_close(db, db64, what + " db")
+
+
+LENS_MIX = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4]
+
+
+@pytest.mark.parametrize("K", [1, 3, 5, 7, 9, 11, 15, 31, 33])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_kernel_sizes(K, dt):
+    print(f"[case] K={K} {dt}", flush=True)
+    _check_case(*_random_case(LENS_MIX, 256, K, dt, dt, seed=K), f"K={K} {dt}")
+
+
+@pytest.mark.parametrize("C", [1, 7, 8, 24, 64, 72, 100, 128, 130, 520, 1000, 1024, 2048, 4104])
+def test_channel_counts(C):
+    """Every lane-slice width (8/4/2/1 channels per lane), partial wave-columns and odd channel counts."""
+    print(f"[case] C={C}", flush=True)
+    _check_case(*_random_case([5, 1, 40, 2, 90, 3], C, 7, torch.bfloat16, torch.bfloat16, seed=C), f"C={C}")
+    _check_case(*_random_case([5, 1, 40, 2, 90, 3], C, 3, torch.float32, torch.float32, seed=C), f"C={C} fp32")
+
+
+@pytest.mark.parametrize("dt,wdt", [(torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16)])
+def test_mixed_activation_and_weight_dtypes(dt, wdt):
+    _check_case(*_random_case(LENS_MIX, 512, 7, dt, wdt, seed=11), f"{dt}/{wdt}")
+
+
+def test_no_bias():
+    _check_case(*_random_case(LENS_MIX, 256, 7, torch.bfloat16, torch.bfloat16, seed=2, bias=False), "no bias")
+
+
+@pytest.mark.parametrize("T", [1, 2, 7, 63, 64, 65, 127, 129, 1000])
+def test_single_sequence_lengths_around_tile_edges(T):
+    _check_case(*_random_case([T], 256, 7, torch.bfloat16, torch.bfloat16, seed=T), f"T={T}")
+
+
+def test_empty_batch():
+    x = torch.empty((0, 64), dtype=torch.bfloat16, device=DEV)
+    cu = torch.zeros(1, dtype=torch.int32, device=DEV)
+    w = torch.randn(64, 7, device=DEV).bfloat16()
+    y = npa.varlen_dwconv_fwd(x, cu, w, None)
+    dx, dw, db = npa.varlen_dwconv_bwd(x, x.clone(), cu, w)
+    torch.cuda.synchronize()
+    assert y.shape == (0, 64) and dx.shape == (0, 64)
+    assert float(dw.abs().max()) == 0.0 and float(db.abs().max()) == 0.0
+
+
+def test_unaligned_views_take_a_narrower_lane_slice():
+    """Row slices that start 2 bytes off a 16-byte boundary must still be computed correctly."""
+    x, cu, w, b, dy = _random_case([33, 90, 5], 264, 7, torch.bfloat16, torch.bfloat16, seed=4)
+    y64 = O.c_oracle_fwd(x, cu, w, b)
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
+    T, C = x.shape
+    for off in (1, 2, 4):
+        bx = torch.zeros(T * C + 8, dtype=torch.bfloat16, device=DEV)
+        bg = torch.zeros(T * C + 8, dtype=torch.bfloat16, device=DEV)
+        xv = bx[off:off + T * C].view(T, C)
+        gv = bg[off:off + T * C].view(T, C)
+        xv.copy_(x)
+        gv.copy_(dy)
+        assert xv.data_ptr() % 16 == 2 * off
+        y = npa.varlen_dwconv_fwd(xv, cu.to(DEV), w.to(DEV), b.to(DEV))
+        dx, dw, db = npa.varlen_dwconv_bwd(xv, gv, cu.to(DEV), w.to(DEV))
+        assert_act_close(y, y64, x.dtype, f"offset {off} y")
+        assert_act_close(dx, dx64, x.dtype, f"offset {off} dx")
+        assert_red_close(dw, dw64, f"offset {off} dw")
+        assert_red_close(db, db64, f"offset {off} db")
+
+
+# ---- boundaries -----------------------------------------------------------------------------------
+def test_nothing_leaks_across_sequences_even_nan_and_inf():
+    x, cu, w, b, dy = _random_case([5, 3, 1, 12, 2, 200, 1, 1, 30], 256, 7, torch.bfloat16, torch.bfloat16, seed=9)
+    cul = cu.tolist()
+    xd, cud, wd, bd, dyd = (t.to(DEV) for t in (x, cu, w, b, dy))
+    y0 = npa.varlen_dwconv_fwd(xd, cud, wd, bd)
+    dx0, _, _ = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    for seq in (3, 5, 6):
+        s, e = cul[seq], cul[seq + 1]
+        x2, dy2 = xd.clone(), dyd.clone()
+        x2[s:e] = float("nan")
+        dy2[s:e] = float("inf")
+        y2 = npa.varlen_dwconv_fwd(x2, cud, wd, bd)
+        dx2, _, _ = npa.varlen_dwconv_bwd(x2, dy2, cud, wd)
+        keep = torch.ones(x.shape[0], dtype=torch.bool, device=DEV)
+        keep[s:e] = False
+        assert torch.equal(y0[keep], y2[keep]), f"forward leaked out of sequence {seq}"
+        assert torch.equal(dx0[keep], dx2[keep]), f"dx leaked out of sequence {seq}"
+        assert bool(torch.isnan(y2[s:e]).all())
+
+
+def test_static_packed_cu_seqlens():
+    """cu_seqlens padded to a fixed length as the static-shape collator emits it (collator.py:430-450):
+    pad pseudo-sequences after the real ones, then zero-length entries equal to F."""
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(20, 129, (37,), generator=g)
+    real_cu = cu_from_lengths(lens)
+    T_real = int(real_cu[-1])
+    F, W = 4096, 128
+    assert T_real < F
+    cu = static_packed_cu(real_cu, F, W, cu_len=96)
+    assert int(cu[-1]) == F and int((cu[1:] == cu[:-1]).sum()) > 5
+    x = torch.randn(F, 256, generator=g).bfloat16()
+    dy = torch.randn(F, 256, generator=g).bfloat16()
+    w = (torch.randn(256, 7, generator=g) * 7 ** -0.5).bfloat16()
+    b = (torch.randn(256, generator=g) * 0.02).bfloat16()
+    _check_case(x, cu, w, b, dy, "static-packed cu")
+    npa.check_cu_seqlens(cu.to(DEV), F)
+
+
+def test_check_cu_seqlens_reports_malformed_input():
+    with pytest.raises(RuntimeError, match="cu_seqlens"):
+        npa.check_cu_seqlens(torch.tensor([0, 5, 3, 9], dtype=torch.int32, device=DEV), 9)
+    with pytest.raises(RuntimeError, match="cu_seqlens"):
+        npa.check_cu_seqlens(torch.tensor([0, 5, 9], dtype=torch.int32, device=DEV), 10)
+    npa.check_cu_seqlens(torch.tensor([0, 5, 5, 9], dtype=torch.int32, device=DEV), 9)
+
+
+def test_malformed_cu_seqlens_cannot_fault():
+    """cu is used only to mask taps: decreasing / out-of-range entries give garbage values, not faults."""
+    x = torch.randn(300, 256, device=DEV).bfloat16()
+    w = torch.randn(256, 7, device=DEV).bfloat16()
+    for bad in ([0, 500, 20, 10 ** 9, -5, 300], [7, 100], [0], [0, 100]):
+        cu = torch.tensor(bad, dtype=torch.int32, device=DEV)
+        y = npa.varlen_dwconv_fwd(x, cu, w, None)
+        dx, dw, db = npa.varlen_dwconv_bwd(x, x, cu, w)
+        torch.cuda.synchronize()
+        assert y.shape == x.shape and dx.shape == x.shape
+
+
+# ---- launch geometry --------------------------------------------------------------------------------
+@pytest.mark.parametrize("tile_rows,bt,nbt,remap", [(8, 1, 1, 2), (16, 2, 3, 2), (64, 4, 8, 1), (128, 2, 16, 1),
+                                                    (40, 1, 64, 1), (256, 4, 200, 2)])
+def test_results_do_not_depend_on_launch_geometry(tile_rows, bt, nbt, remap):
+    """y and dx are bit-identical for any tiling; dw/db differ only by summation order."""
+    wl, y64, dx64, dw64, db64 = workload_with_oracle(5, 9000, 1024)
+    d = wl.to(DEV)
+    y0, dx0, dw0, db0 = _run_all(d)
+    tf = _lib.Tuning(tile_rows=tile_rows, bt=bt, nbt=nbt, xcd_remap=remap)
+    y = npa.varlen_dwconv_fwd(d.x, d.cu_seqlens, d.weight, d.bias, tuning=tf)
+    dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, tuning=tf)
+    assert torch.equal(y, y0) and torch.equal(dx, dx0)
+    assert_red_close(dw, dw64, "dw")
+    assert_red_close(db, db64, "db")
+    torch.testing.assert_close(dw, dw0, rtol=1e-5, atol=1e-3)
+
+
+def test_backward_outputs_can_be_requested_separately():
+    wl, y64, dx64, dw64, db64 = workload_with_oracle(5, 9000, 1024)
+    d = wl.to(DEV)
+    _, dx0, dw0, db0 = _run_all(d)
+    dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, need_dw=False)
+    assert dw is None and db is None and torch.equal(dx, dx0)
+    dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, need_dx=False)
+    assert dx is None and torch.equal(dw, dw0) and torch.equal(db, db0)
+
+
+def test_workspace_contents_do_not_matter():
+    wl, *_ = workload_with_oracle(5, 9000, 1024)
+    d = wl.to(DEV)
+    _, _, dw0, db0 = _run_all(d)
+    n = npa.bwd_workspace_bytes(wl.T, wl.C, wl.K, wl.dtype)
+    ws = torch.full((n,), 0xFF, dtype=torch.uint8, device=DEV)   # NaN bit patterns everywhere
+    _, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, workspace=ws)
+    assert torch.equal(dw, dw0) and torch.equal(db, db0)
+    with pytest.raises(RuntimeError, match="workspace"):
+        npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, workspace=ws[: n // 2])
+
+
+# ---- size-independent properties at the headline size -------------------------------------------------
+def test_linearity_and_adjoint_identity_at_full_size():
+    wl = make_workload(3).to(DEV)
+    x, cu, w, dy = wl.x, wl.cu_seqlens, wl.weight, wl.dy
+    y = npa.varlen_dwconv_fwd(x, cu, w, None)
+    dx, dw, db = npa.varlen_dwconv_bwd(x, dy, cu, w)
+    # <conv(x), dy> = <x, dx> = <w, dw>, each side accumulated in fp64 on the device. y and dx carry
+    # one bf16 rounding per element (relative 2^-9, random sign), so the sums agree to ~1e-4 relative.
+    lhs = (y.double() * dy.double()).sum()
+    mid = (x.double() * dx.double()).sum()
+    rhs = (w.double() * dw.double()).sum()
+    scale = float((y.double().abs() * dy.double().abs()).sum())
+    assert abs(float(lhs - mid)) <= 1e-4 * scale and abs(float(lhs - rhs)) <= 1e-4 * scale
+    torch.testing.assert_close(db.double(), dy.double().sum(0), rtol=1e-6, atol=1e-3)
+    # scaling x by 2 (exact in bf16) scales y and dw exactly by 2
+    y2 = npa.varlen_dwconv_fwd(x * 2, cu, w, None)
+    assert torch.equal(y2, y * 2)
+    _, dw2, _ = npa.varlen_dwconv_bwd(x * 2, dy, cu, w, need_dx=False)
+    assert torch.equal(dw2, dw * 2)
