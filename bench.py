@@ -1,0 +1,243 @@
+#!/usr/bin/env python3
+"""Benchmark of the varlen depthwise conv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 3] [--no-cpu-baseline]
+
+A step is one forward plus one backward (dx, dweight, dbias) of the configured workload through the
+C ABI of libnplm_dwconv.so, with every input already resident in HBM. The default workload is
+configuration 3 of nanoplm_amd.workloads (T=131072 packed tokens, C=1024, K=7, bf16), the one the
+headline metric is quoted on. Three input/output sets (> 256 MB each) are rotated so no step reads
+a tensor that is still in the Infinity Cache.
+
+One JSON line is printed:
+  value         tokens/s over the K timed steps (wall clock, stream synchronised on both sides)
+  roofline      the dominant kernel (the fused backward): algorithmic bytes per launch divided by its
+                average duration, measured with HIP events recorded on the launch stream
+  roofline_fwd  the same for the forward kernel (informational)
+  cpu_baseline  the reference path (per-sequence torch conv1d + autograd, oracle/dwconv_ref.py) timed
+                on this box's host cores on a bounded sample of the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and
+# scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
+# profiles/): keyed by (workload name, kernel).
+MEASURED_TRAFFIC = {}
+
+
+def _hip():
+    lib = ctypes.CDLL("libamdhip64.so")
+    lib.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    lib.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    lib.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+    lib.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    return lib
+
+
+class HipEvents:
+    """Raw HIP events on a given stream (torch.cuda.Event only sees torch's current stream)."""
+
+    def __init__(self, n):
+        self.hip = _hip()
+        self.ev = []
+        for _ in range(n):
+            e = ctypes.c_void_p()
+            rc = self.hip.hipEventCreate(ctypes.byref(e))
+            if rc:
+                raise RuntimeError(f"hipEventCreate failed: {rc}")
+            self.ev.append(e)
+
+    def record(self, i, stream):
+        rc = self.hip.hipEventRecord(self.ev[i], ctypes.c_void_p(stream))
+        if rc:
+            raise RuntimeError(f"hipEventRecord failed: {rc}")
+
+    def elapsed_us(self, i, j):
+        self.hip.hipEventSynchronize(self.ev[j])
+        ms = ctypes.c_float()
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), self.ev[i], self.ev[j])
+        if rc:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return ms.value * 1e3
+
+
+def cpu_baseline(wl, sample_tokens):
+    """Reference path on the host cores, on the first sequences of the workload (about sample_tokens rows)."""
+    import torch
+    from oracle.dwconv_ref import ref_dwconv_varlen_grads
+
+    cu = wl.cu_seqlens
+    n = int(torch.searchsorted(cu, torch.tensor(sample_tokens, dtype=cu.dtype)).item())
+    n = max(1, min(n, cu.numel() - 1))
+    Ts = int(cu[n])
+    x, dy, cus = wl.x[:Ts], wl.dy[:Ts], cu[: n + 1]
+    threads = torch.get_num_threads()
+
+    def run(dtype):
+        ref_dwconv_varlen_grads(x, cus, wl.weight, wl.bias, dy, dtype)      # warm-up
+        ts = []
+        for _ in range(3):
+            t = time.perf_counter()
+            ref_dwconv_varlen_grads(x, cus, wl.weight, wl.bias, dy, dtype)
+            ts.append(time.perf_counter() - t)
+        return statistics.median(ts)
+
+    t_bf16 = run(wl.dtype)
+    t_f32 = run(torch.float32)
+    return {
+        "value": Ts / t_bf16, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": f"first {n} sequences ({Ts} of {wl.T} tokens) of {wl.name}, fwd+bwd via per-sequence "
+                  f"torch conv1d + autograd in {str(wl.dtype).replace('torch.', '')}, median of 3 after 1 warm-up",
+        "seconds_per_pass": t_bf16,
+        "fp32_tokens_per_s": Ts / t_f32,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1); "
+                 "the op shards at sequence boundaries or along channels without communication.")
+
+    import torch
+    import nanoplm_amd as npa
+    from nanoplm_amd import _lib
+    from nanoplm_amd.workloads import make_workload
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a ROCm GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+
+    wl = make_workload(args.config, with_dy=True)
+    d = wl.to(dev)
+    T, C, K, S = wl.T, wl.C, wl.K, wl.S
+    fwd_bwd = wl.passes == "fwd+bwd"
+    NSET = 3
+    xs = [d.x] + [torch.randn(T, C, device=dev).to(wl.dtype) for _ in range(NSET - 1)]
+    gs = [d.dy] + [torch.randn(T, C, device=dev).to(wl.dtype) for _ in range(NSET - 1)]
+    ys = [torch.empty_like(d.x) for _ in range(NSET)]
+    dxs = [torch.empty_like(d.x) for _ in range(NSET)]
+    dw = torch.empty((C, K), dtype=torch.float32, device=dev)
+    db = torch.empty((C,), dtype=torch.float32, device=dev)
+    act = _lib.BF16 if wl.dtype == torch.bfloat16 else _lib.F32
+    ws_bytes = int(lib.nplm_dwconv_bwd_workspace_bytes(T, C, K, act))
+    ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    cu, w, b = d.cu_seqlens, d.weight, d.bias
+    tune = _lib.Tuning()
+
+    def fwd(i):
+        j = i % NSET
+        _lib.check(lib.nplm_dwconv_fwd(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(), ys[j].data_ptr(),
+                                       T, C, K, S, act, act, stream), "nplm_dwconv_fwd")
+
+    def bwd(i, t=None):
+        j = i % NSET
+        args_ = (xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(),
+                 db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act, stream)
+        rc = lib.nplm_dwconv_bwd(*args_) if t is None else lib.nplm_dwconv_bwd_tuned(*args_, t)
+        _lib.check(rc, "nplm_dwconv_bwd")
+
+    def step(i):
+        fwd(i)
+        if fwd_bwd:
+            bwd(i)
+
+    # ---- whole-step throughput -----------------------------------------------------------------
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tokens_per_s = T / (ms_per_step / 1e3)
+
+    # ---- per-kernel durations with HIP events on the launch stream ---------------------------------
+    n_ev = min(max(args.steps, 10), 100)
+    ev = HipEvents(4)
+    tune.mid_event = ev.ev[2]
+    fwd_us, bwd_us, fin_us = [], [], []
+    for i in range(n_ev):
+        ev.record(0, stream)
+        fwd(i)
+        ev.record(1, stream)
+        if fwd_bwd:
+            bwd(i, tune)            # records event 2 between the fused kernel and the finalize kernel
+            ev.record(3, stream)
+        torch.cuda.synchronize()
+        fwd_us.append(ev.elapsed_us(0, 1))
+        if fwd_bwd:
+            bwd_us.append(ev.elapsed_us(1, 2))
+            fin_us.append(ev.elapsed_us(2, 3))
+    fwd_avg = statistics.fmean(fwd_us)
+    fwd_bytes = wl.algorithmic_bytes("fwd")
+
+    def roof(nbytes, us, kernel):
+        gbps = nbytes / us / 1e3
+        return {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                "traffic": MEASURED_TRAFFIC.get((wl.name, kernel)), "kernel": kernel, "avg_us": us,
+                "algorithmic_bytes": nbytes}
+
+    out = {
+        "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
+                  if args.config == 3 else f"varlen dwconv {wl.passes} tokens/s ({wl.name})",
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
+        "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
+        "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
+                   "rotating_sets": NSET},
+        "step_algorithmic_bytes": wl.algorithmic_bytes(),
+        "step_GBps": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9,
+        "step_frac_of_hbm_peak": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+    }
+    if fwd_bwd:
+        out["roofline"] = roof(wl.algorithmic_bytes("bwd"), statistics.fmean(bwd_us), "dwconv_bwd_kernel")
+        out["roofline_fwd"] = roof(fwd_bytes, fwd_avg, "dwconv_fwd_lds_kernel")
+        out["finalize_avg_us"] = statistics.fmean(fin_us)
+    else:
+        out["roofline"] = roof(fwd_bytes, fwd_avg, "dwconv_fwd_lds_kernel")
+
+    # ---- what a plain copy reaches on this box (context for the roofline fraction) ----------------
+    cp_us = []
+    for i in range(20):
+        ev.record(0, stream)
+        _lib.check(lib.nplm_dwconv_debug_copy(xs[i % NSET].data_ptr(), ys[i % NSET].data_ptr(),
+                                              T * C * d.x.element_size(), stream), "nplm_dwconv_debug_copy")
+        ev.record(1, stream)
+        torch.cuda.synchronize()
+        cp_us.append(ev.elapsed_us(0, 1))
+    out["plain_copy_GBps"] = 2 * T * C * d.x.element_size() / statistics.median(cp_us[2:]) / 1e3
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, args.cpu_sample_tokens)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -31,7 +31,8 @@ class Tuning(ctypes.Structure):
     """Mirror of ``nplm_dwconv_tuning`` (csrc/dwconv_internal.h); 0 keeps the library default."""
 
     _fields_ = [(n, ctypes.c_int32) for n in
-                ("vec", "unroll", "tile_rows", "bw", "bt", "nbt", "xcd_remap", "maxt")]
+                ("vec", "unroll", "tile_rows", "bw", "bt", "nbt", "xcd_remap", "maxt", "algo", "nwl", "reserved")
+                ] + [("mid_event", ctypes.c_void_p)]
 
 
 def load():
@@ -65,6 +66,8 @@ def load():
     lib.nplm_dwconv_bwd_slabs.restype = i32
     lib.nplm_dwconv_debug_intervals.argtypes = [vp, i32, i64, i64, i64, i64, vp, vp]
     lib.nplm_dwconv_debug_intervals.restype = i64
+    lib.nplm_dwconv_debug_copy.argtypes = [vp, vp, sz, vp]
+    lib.nplm_dwconv_debug_copy.restype = ctypes.c_int
     lib.nplm_dwconv_check_cu.argtypes = [vp, i32, i64, vp]
     lib.nplm_dwconv_check_cu.restype = ctypes.c_int
     _lib = lib

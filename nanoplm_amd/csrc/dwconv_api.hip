@@ -67,9 +67,13 @@ int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bi
     p.unroll = tune->unroll > 0 ? tune->unroll : default_unroll(bwd, K, p.vec);
     p.maxt = tune->maxt > 0 ? tune->maxt : default_maxt(bwd, K, p.vec);
     if (p.maxt < 64 || p.maxt > 1024 || p.maxt % 64) return -NPLM_DWCONV_ETUNING;
-    int R = tune->tile_rows > 0 ? tune->tile_rows : 64;
+    int R = tune->tile_rows > 0 ? tune->tile_rows : (bwd ? 128 : 64);
     if (R > kMaxTileRows || p.unroll > 64) return -NPLM_DWCONV_ETUNING;
     R = ceil_div(R, p.unroll) * p.unroll;
+    // row offsets inside a tile are 32-bit byte offsets
+    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
+    while ((long long)(R + K) * row_bytes >= INT_MAX && R > p.unroll) R = ceil_div(R / 2, p.unroll) * p.unroll;
+    if ((long long)(R + K) * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
     p.R = R;
     p.ntiles = ceil_div(T, R);
     p.ncols = C / p.vec;
@@ -91,17 +95,20 @@ int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bi
         if (tune->nbt <= 0 && nbt > cap) nbt = (int)cap;
     }
     if (nbt < 1) nbt = 1;
-    // keep the grid a multiple of the XCD count when it is large enough, so the remap applies
+    // keep the grid a multiple of the XCD count when it is large enough: every XCD gets equal work
     if (tune->nbt <= 0 && nbt >= kNumXCD) nbt -= nbt % kNumXCD;
     p.nbt = nbt;
-    p.remap = (tune->xcd_remap != 2) && ((long long)p.ncb * p.nbt) % kNumXCD == 0;
+    p.remap = (tune->xcd_remap == 1) && ((long long)p.ncb * p.nbt) % kNumXCD == 0;
     *out = p;
     return 0;
 }
 
-void fill_args(const Plan& p, ConvArgs* a) {
-    a->R = p.R; a->ntiles = p.ntiles; a->ncols = p.ncols; a->nwc = p.nwc;
-    a->bw = p.bw; a->bt = p.bt; a->ncb = p.ncb; a->nbt = p.nbt; a->xcd_remap = p.remap;
+Geo make_geo(const Plan& p, long long T, int C, int S, int w_bf16) {
+    Geo g{};
+    g.T = (int32_t)T; g.C = C; g.S = S; g.w_bf16 = w_bf16;
+    g.R = p.R; g.ntiles = p.ntiles; g.ncols = p.ncols; g.nwc = p.nwc;
+    g.bw = p.bw; g.bt = p.bt; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_remap = p.remap;
+    return g;
 }
 
 int check_common(long long T, int C, int K, int S, int act_dtype, int w_dtype) {
@@ -114,28 +121,131 @@ int check_common(long long T, int C, int K, int S, int act_dtype, int w_dtype) {
     return 0;
 }
 
-hipError_t launch_fwd(int K, bool bf16, const Plan& p, const ConvArgs& a, dim3 grid, dim3 block, hipStream_t s) {
+hipError_t launch_fwd(int K, bool bf16, const Plan& p, const ConvPtrs& a, const Geo& g, hipStream_t s) {
+    const dim3 grid(p.ncb * p.nbt), block(p.bw * p.bt * 64);
     switch (K) {
-        case 3: return launch_fwd_k3(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
-        case 5: return launch_fwd_k5(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
-        case 7: return launch_fwd_k7(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
-        case 9: return launch_fwd_k9(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
-        case 15: return launch_fwd_k15(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
-        case 31: return launch_fwd_k31(bf16, p.vec, p.unroll, p.maxt, a, grid, block, s);
+        case 3: return launch_fwd_k3(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
+        case 5: return launch_fwd_k5(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
+        case 7: return launch_fwd_k7(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
+        case 9: return launch_fwd_k9(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
+        case 15: return launch_fwd_k15(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
+        case 31: return launch_fwd_k31(bf16, p.vec, p.unroll, p.maxt, a, g, grid, block, s);
     }
     return hipErrorInvalidConfiguration;
 }
-hipError_t launch_bwd(int K, bool bf16, const Plan& p, const ConvArgs& a, dim3 grid, dim3 block, size_t shmem,
+hipError_t launch_bwd(int K, bool bf16, const Plan& p, bool wdx, bool wdw, const ConvPtrs& a, const Geo& g,
                       hipStream_t s) {
+    const dim3 grid(p.ncb * p.nbt), block(p.bw * p.bt * 64);
+    const size_t shmem = (size_t)p.bw * p.bt * p.vec * 64 * sizeof(float);
     switch (K) {
-        case 3: return launch_bwd_k3(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
-        case 5: return launch_bwd_k5(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
-        case 7: return launch_bwd_k7(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
-        case 9: return launch_bwd_k9(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
-        case 15: return launch_bwd_k15(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
-        case 31: return launch_bwd_k31(bf16, p.vec, p.unroll, p.maxt, a, grid, block, shmem, s);
+        case 3: return launch_bwd_k3(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
+        case 5: return launch_bwd_k5(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
+        case 7: return launch_bwd_k7(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
+        case 9: return launch_bwd_k9(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
+        case 15: return launch_bwd_k15(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
+        case 31: return launch_bwd_k31(bf16, p.vec, p.unroll, p.maxt, wdx, wdw, a, g, grid, block, shmem, s);
     }
     return hipErrorInvalidConfiguration;
+}
+
+// ---- LDS-staged pipelined kernels ---------------------------------------------------------------
+constexpr size_t kLdsBytesPerCU = 160u << 10;
+
+struct LdsPlan {
+    LdsShapeSel sh;
+    int R, ntiles, ncb, nbt;
+};
+
+// Whether the LDS kernels can take this problem at all (16-byte row granularity, built kernel size).
+bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    const int E = bf16 ? 2 : 4;
+    if (!lds_kernel_size(K) || T < 1) return false;
+    if (((long long)C * E) % 16 || align_bits % 16) return false;
+    return (long long)C * E >= 1024;   // narrower rows leave most of a block idle: sliding-window kernels
+}
+
+int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
+    LdsPlan p{};
+    nplm_dwconv_tuning z{};
+    if (!tune) tune = &z;
+    const int E = bf16 ? 2 : 4;
+    p.sh = lds_default_shape(bwd, bf16);
+    if (tune->vec > 0) p.sh.vec = tune->vec;
+    if (tune->unroll > 0) p.sh.rw = tune->unroll;
+    if (tune->bt > 0) p.sh.nrg = tune->bt;
+    if (tune->bw > 0) p.sh.ncw = tune->bw;
+    if (tune->nwl > 0) p.sh.nwl = tune->nwl;
+    const long long cb_bytes = (long long)p.sh.ncw * 64 * p.sh.vec * E;
+    const long long row_bytes = (long long)C * E;
+    p.R = p.sh.rw * p.sh.nrg;
+    const size_t shmem = (size_t)(bwd ? 4 : 2) * (p.R + K - 1) * cb_bytes;
+    if (shmem > kLdsBytesPerCU || cb_bytes % 1024) return -NPLM_DWCONV_ETUNING;
+    if ((long long)(p.R + K) * row_bytes + row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
+    p.ncb = ceil_div(row_bytes, cb_bytes);
+    p.ntiles = ceil_div(T, p.R);
+    int nbt = tune->nbt > 0 ? tune->nbt : kNumCU / p.ncb;
+    if (nbt < 1) nbt = 1;
+    if (nbt > p.ntiles) nbt = p.ntiles;
+    if (bwd && tune->nbt <= 0) {
+        const size_t slab = (size_t)(K + 1) * C * sizeof(float);
+        const long long cap = (long long)(kSlabBudgetBytes / slab);
+        if (nbt > cap && cap >= 1) nbt = (int)cap;
+    }
+    p.nbt = nbt;
+    *out = p;
+    return 0;
+}
+
+LdsGeo make_lds_geo(const LdsPlan& p, long long T, int C, int S, int w_bf16) {
+    LdsGeo g{};
+    g.T = (int32_t)T; g.C = C; g.S = S; g.w_bf16 = w_bf16;
+    g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt;
+    return g;
+}
+
+hipError_t launch_fwd_lds(int K, const LdsPlan& p, const ConvPtrs& a, const LdsGeo& g, hipStream_t s) {
+    const dim3 grid(p.ncb * p.nbt);
+    switch (K) {
+        case 3: return launch_fwd_lds_k3(p.sh, a, g, grid, s);
+        case 5: return launch_fwd_lds_k5(p.sh, a, g, grid, s);
+        case 7: return launch_fwd_lds_k7(p.sh, a, g, grid, s);
+        case 9: return launch_fwd_lds_k9(p.sh, a, g, grid, s);
+    }
+    return hipErrorInvalidConfiguration;
+}
+hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const ConvPtrs& a, const LdsGeo& g,
+                          hipStream_t s) {
+    const dim3 grid(p.ncb * p.nbt);
+    switch (K) {
+        case 3: return launch_bwd_lds_k3(p.sh, wdx, wdw, a, g, grid, s);
+        case 5: return launch_bwd_lds_k5(p.sh, wdx, wdw, a, g, grid, s);
+        case 7: return launch_bwd_lds_k7(p.sh, wdx, wdw, a, g, grid, s);
+        case 9: return launch_bwd_lds_k9(p.sh, wdx, wdw, a, g, grid, s);
+    }
+    return hipErrorInvalidConfiguration;
+}
+
+// algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged.
+// Measured on MI355X at T=131072, C=1024, K=7, bf16: the forward is fastest LDS-staged; the backward
+// keeps two tensors with halos in flight, which LDS (160 KiB per CU) cannot hold twice over, so the
+// register-resident sliding-window kernel wins there.
+int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    const bool ok = lds_eligible(bf16, T, C, K, align_bits);
+    if (tune && tune->algo == 2) return ok ? 2 : -NPLM_DWCONV_ETUNING;
+    if (tune && tune->algo == 1) return 1;
+    return (ok && !bwd) ? 2 : 1;
+}
+
+// 256 threads x 4 x 16 B = one contiguous 16 KiB chunk per block
+__global__ void __launch_bounds__(256) copy_chunks_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, size_t nvec) {
+    const size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + u * 256 < nvec) v[u] = src[base + u * 256];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + u * 256 < nvec) dst[base + u * 256] = v[u];
 }
 
 __global__ void fill_zero_kernel(float* p, long long n) {
@@ -161,10 +271,21 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
     if (bits % E) return -NPLM_DWCONV_EALIGN;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
+    hipStream_t s = (hipStream_t)stream;
+    const int algo = choose_algo(false, tune, bf16, T, C, K, bits);
+    if (algo < 0) return algo;
+    if (algo == 2) {
+        LdsPlan lp;
+        rc = make_lds_plan(false, bf16, T, C, K, tune, &lp);
+        if (rc) return rc;
+        const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
+        const hipError_t e = launch_fwd_lds(K, lp, la, make_lds_geo(lp, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
+        if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
+        return (int)e;
+    }
     Plan p;
     rc = make_plan(false, bf16, T, C, K, bits, tune, &p);
     if (rc) return rc;
-    hipStream_t s = (hipStream_t)stream;
     if (p.generic) {
         const int wpb = 4;
         int blocks = ceil_div(T, wpb);
@@ -177,11 +298,8 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
                                (int)T, C, S, K, (int)(w_dtype == NPLM_DWCONV_BF16), 0);
         return (int)hipGetLastError();
     }
-    ConvArgs a{};
-    a.x = x; a.dy = nullptr; a.cu = cu; a.w = w; a.b = b; a.out = y; a.partial = nullptr;
-    a.T = (int32_t)T; a.C = C; a.S = S; a.K = K; a.w_bf16 = (w_dtype == NPLM_DWCONV_BF16);
-    fill_args(p, &a);
-    const hipError_t e = launch_fwd(K, bf16, p, a, dim3(p.ncb * p.nbt), dim3(p.bw * p.bt * 64), s);
+    const ConvPtrs a{x, nullptr, cu, w, b, y, nullptr};
+    const hipError_t e = launch_fwd(K, bf16, p, a, make_geo(p, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
     if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
     return (int)e;
 }
@@ -207,6 +325,36 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
 
+    const int algo = choose_algo(true, tune, bf16, T, C, K, bits);
+    if (algo < 0) return algo;
+    if (algo == 2) {
+        LdsPlan lp;
+        rc = make_lds_plan(true, bf16, T, C, K, tune, &lp);
+        if (rc) return rc;
+        const size_t slab_bytes = (size_t)(K + 1) * C * sizeof(float);
+        float* part = nullptr;
+        if (want_red) {
+            if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab_bytes * (size_t)lp.nbt)
+                return -NPLM_DWCONV_EWORKSPACE;
+            part = reinterpret_cast<float*>(workspace);
+        }
+        const ConvPtrs la{x, dy, cu, w, nullptr, dx, part};
+        hipError_t e = launch_bwd_lds(K, lp, dx != nullptr, want_red, la,
+                                      make_lds_geo(lp, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
+        if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
+        if (e != hipSuccess) return (int)e;
+        if (tune && tune->mid_event) {
+            e = hipEventRecord((hipEvent_t)tune->mid_event, s);
+            if (e != hipSuccess) return (int)e;
+        }
+        if (want_red) {
+            const long long n_out = (long long)(K + 1) * C;
+            hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)),
+                               dim3(64 * FIN_SPLIT), 0, s, (const float*)part, lp.nbt, C, K, dw, db);
+            e = hipGetLastError();
+        }
+        return (int)e;
+    }
     Plan p;
     rc = make_plan(true, bf16, T, C, K, bits, tune, &p);
     if (rc) return rc;
@@ -256,14 +404,13 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
             if (e != hipSuccess) return (int)e;
         }
     } else {
-        ConvArgs a{};
-        // dx-only calls never touch x; point it at dy so the loads stay valid
-        a.x = x ? x : dy; a.dy = dy; a.cu = cu; a.w = w; a.b = nullptr; a.out = dx; a.partial = partial;
-        a.T = (int32_t)T; a.C = C; a.S = S; a.K = K; a.w_bf16 = w_bf16;
-        fill_args(p, &a);
-        const size_t shmem = (size_t)p.bw * p.bt * p.vec * 64 * sizeof(float);
-        const hipError_t e = launch_bwd(K, bf16, p, a, dim3(p.ncb * p.nbt), dim3(p.bw * p.bt * 64), shmem, s);
+        const ConvPtrs a{x, dy, cu, w, nullptr, dx, partial};
+        const hipError_t e = launch_bwd(K, bf16, p, dx != nullptr, want_red, a, make_geo(p, T, C, S, w_bf16), s);
         if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
+        if (e != hipSuccess) return (int)e;
+    }
+    if (tune && tune->mid_event) {
+        const hipError_t e = hipEventRecord((hipEvent_t)tune->mid_event, s);
         if (e != hipSuccess) return (int)e;
     }
     if (want_red) {
@@ -314,16 +461,25 @@ int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const
 
 size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     Plan p;
-    if (make_plan(true, act_dtype == NPLM_DWCONV_BF16, T, C, K, 0, nullptr, &p)) return 0;
+    if (make_plan(true, bf16, T, C, K, 0, nullptr, &p)) return 0;
     const size_t bytes = (size_t)p.nbt * (K + 1) * C * sizeof(float);
     return (bytes + 255) & ~(size_t)255;
 }
 
 int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const int algo = choose_algo(true, tune, bf16, T, C, K, 0);
+    if (algo < 0) return 0;
+    if (algo == 2) {
+        LdsPlan lp;
+        if (make_lds_plan(true, bf16, T, C, K, tune, &lp)) return 0;
+        return lp.nbt;
+    }
     Plan p;
-    if (make_plan(true, act_dtype == NPLM_DWCONV_BF16, T, C, K, 0, tune, &p)) return 0;
+    if (make_plan(true, bf16, T, C, K, 0, tune, &p)) return 0;
     return p.nbt;
 }
 
@@ -340,6 +496,16 @@ int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, cons
                           const nplm_dwconv_tuning* tune) {
     return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, stream,
                     tune);
+}
+
+int nplm_dwconv_debug_copy(const void* src, void* dst, size_t bytes, void* stream) {
+    if (!src || !dst) return -NPLM_DWCONV_ENULL;
+    if (bytes % 16 || ((uintptr_t)src | (uintptr_t)dst) % 16) return -NPLM_DWCONV_EALIGN;
+    if (bytes == 0) return 0;
+    const size_t nvec = bytes / 16;
+    hipLaunchKernelGGL(copy_chunks_kernel, dim3((unsigned)((nvec + 1023) / 1024)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4*)src, (u32x4*)dst, nvec);
+    return (int)hipGetLastError();
 }
 
 int64_t nplm_dwconv_debug_intervals(const int32_t* cu_host, int32_t S, int64_t T, int64_t start, int64_t step,

@@ -33,6 +33,28 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Buffer addressing. Row slices are moved with MUBUF instructions: address = descriptor base +
+// scalar byte offset (the row, wave-uniform) + per-lane byte offset (the channel slice, constant for
+// the whole kernel), so no vector ALU work goes into address arithmetic.
+// ---------------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Raw (untyped, stride 0) buffer descriptor over `bytes` bytes at `base`; 0x00020000 = 32-bit data
+// format word of gfx9-family descriptors.
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+// Descriptor over rows [row0, T) of a [T, row_bytes] tensor (capped at 4 GiB - 1).
+__device__ __forceinline__ rsrc_t rows_rsrc(const void* tensor, int row0, int T, size_t row_bytes) {
+    const size_t rem = (size_t)(T - row0) * row_bytes;
+    const uint32_t n = rem > 0xffffffffull ? 0xffffffffu : (uint32_t)rem;
+    return make_rsrc(reinterpret_cast<const char*>(tensor) + (size_t)row0 * row_bytes, n);
+}
+
+// ---------------------------------------------------------------------------------------------
 // RowVec: VEC adjacent channels of one row, as stored in memory.
 // ---------------------------------------------------------------------------------------------
 template <bool BF16, int VEC> struct RowVec;
@@ -53,6 +75,16 @@ template <int VEC> struct RowVec<true, VEC> {
         else if constexpr (NDW == 2) { *reinterpret_cast<uint2*>(p) = make_uint2(d[0], d[1]); }
         else { *reinterpret_cast<uint32_t*>(p) = d[0]; }
     }
+    __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) {
+        if constexpr (NDW == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w; }
+        else if constexpr (NDW == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); d[0] = t.x; d[1] = t.y; }
+        else { d[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0); }
+    }
+    __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const {
+        if constexpr (NDW == 4) { u32x4 t = {d[0], d[1], d[2], d[3]}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, 0); }
+        else if constexpr (NDW == 2) { u32x2 t = {d[0], d[1]}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, 0); }
+        else { __builtin_amdgcn_raw_buffer_store_b32(d[0], r, voff, soff, 0); }
+    }
     __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
 #pragma unroll
         for (int i = 0; i < NDW; ++i) { f[2 * i] = bf16_lo(d[i]); f[2 * i + 1] = bf16_hi(d[i]); }
@@ -67,6 +99,8 @@ template <> struct RowVec<true, 1> {
     uint16_t h;
     __device__ __forceinline__ void load(const char* p) { h = *reinterpret_cast<const uint16_t*>(p); }
     __device__ __forceinline__ void store(char* p) const { *reinterpret_cast<uint16_t*>(p) = h; }
+    __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) { h = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0); }
+    __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const { __builtin_amdgcn_raw_buffer_store_b16(h, r, voff, soff, 0); }
     __device__ __forceinline__ void to_f32(float (&f)[1]) const { f[0] = bf16_to_f32(h); }
     __device__ __forceinline__ void from_f32(const float (&f)[1]) { h = f32_to_bf16(f[0]); }
 };
@@ -84,6 +118,16 @@ template <int VEC> struct RowVec<false, VEC> {
         if constexpr (VEC == 4) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
         else if constexpr (VEC == 2) { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
         else { *reinterpret_cast<float*>(p) = v[0]; }
+    }
+    __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) {
+        if constexpr (VEC == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w); }
+        else if constexpr (VEC == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); }
+        else { v[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0)); }
+    }
+    __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const {
+        if constexpr (VEC == 4) { u32x4 t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, 0); }
+        else if constexpr (VEC == 2) { u32x2 t = {__float_as_uint(v[0]), __float_as_uint(v[1])}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, 0); }
+        else { __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[0]), r, voff, soff, 0); }
     }
     __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
 #pragma unroll
@@ -104,6 +148,16 @@ template <int VEC> struct RowVec<false, VEC> {
 // kernels read or write out of bounds. Rows below cu[0] or at/after cu[S] fall into one extra
 // pseudo-sequence on that side.
 // ---------------------------------------------------------------------------------------------
+// One entry of cu as a scalar: on the device the value is forced into a scalar register, which keeps
+// the whole cursor (and every comparison against it) off the vector ALU.
+__host__ __device__ __forceinline__ int cu_at(const int32_t* __restrict__ cu, int i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return __builtin_amdgcn_readfirstlane(cu[i]);
+#else
+    return cu[i];
+#endif
+}
+
 struct SeqCursor {
     int seq;  // index of the current interval; -1 / S for the pseudo-sequences at either end
     int cs;   // first row of the interval
@@ -115,11 +169,11 @@ struct SeqCursor {
         // first i in [lo, S) with cu[i+1] > t, else S
         while (lo < hi) {
             int mid = (lo + hi) >> 1;
-            if (cu[mid + 1] > t) hi = mid; else lo = mid + 1;
+            if (cu_at(cu, mid + 1) > t) hi = mid; else lo = mid + 1;
         }
         seq = lo;
-        if (lo < S) { cs = cu[lo]; ce = cu[lo + 1]; }
-        else        { cs = cu[S];  ce = T; }
+        if (lo < S) { cs = cu_at(cu, lo); ce = cu_at(cu, lo + 1); }
+        else        { cs = cu_at(cu, S);  ce = T; }
         if (cs > t) { ce = cs; cs = 0; seq = -1; }   // row lies before cu[0]
     }
     // Move forward until the interval contains row t (t must not decrease between calls).
@@ -127,7 +181,7 @@ struct SeqCursor {
         while (t >= ce && seq < S) {
             ++seq;
             cs = ce;
-            ce = (seq < S) ? cu[seq + 1] : T;
+            ce = (seq < S) ? cu_at(cu, seq + 1) : T;
         }
     }
 };

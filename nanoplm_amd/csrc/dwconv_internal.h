@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "dwconv_kernels.h"
+#include "dwconv_lds_kernels.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -19,9 +20,16 @@ typedef struct nplm_dwconv_tuning {
     int32_t bw;         // wave-columns per block (power of two)
     int32_t bt;         // token slots per block
     int32_t nbt;        // token-blocks in the grid
-    int32_t xcd_remap;  // 1 = on, 2 = off
+    int32_t xcd_remap;  // 1 = give each XCD a contiguous share of the token-blocks (off by default: measured slower)
     int32_t maxt;       // launch-bounds class (threads per block the kernel was compiled for)
+    int32_t algo;       // 1 = sliding-window (register) kernels, 2 = LDS-staged pipelined kernels
+    int32_t nwl;        // LDS kernels: loader waves per block
+    int32_t reserved;
+    void* mid_event;    // backward: hipEvent_t recorded between the fused kernel and the finalize kernel
 } nplm_dwconv_tuning;
+// For algo 2 the fields mean: vec = channels per lane, unroll = rows per wave (RW), bt = row groups
+// per block (tile rows = RW * bt), bw = wave-columns per block, nwl = loader waves, nbt = token
+// blocks; tile_rows, xcd_remap and maxt are ignored. Only shapes the library was built with exist.
 
 // Same contracts as nplm_dwconv_fwd / nplm_dwconv_bwd, with geometry overrides. An override the
 // build does not hold a kernel for yields -NPLM_DWCONV_ETUNING.
@@ -43,19 +51,51 @@ int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype
 int64_t nplm_dwconv_debug_intervals(const int32_t* cu_host, int32_t S, int64_t T, int64_t start, int64_t step,
                                     int64_t relocate_every, int32_t* cs_out, int32_t* ce_out);
 
+// Plain streaming copy of `bytes` bytes (multiple of 16, 16-byte aligned pointers) with one block
+// per contiguous 16 KiB: the measuring stick for what a 1-read-1-write kernel reaches on this GPU and
+// the known-size kernel that calibrates the profiler's HBM byte counters.
+int nplm_dwconv_debug_copy(const void* src, void* dst, size_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
 
 namespace nplm {
 
+// The device pointers of one call (host-side bundle; kernels take them as separate arguments).
+struct ConvPtrs {
+    const void* x;
+    const void* dy;
+    const int32_t* cu;
+    const void* w;
+    const void* b;
+    void* out;        // y (forward) or dx (backward)
+    float* partial;   // backward: dw/db slabs
+};
+
 // One launcher per specialised kernel size, each in its own translation unit.
 // Return hipErrorInvalidConfiguration when the (vec, unroll, maxt) combination is not built.
-#define NPLM_DECLARE_K(KK)                                                                              \
-    hipError_t launch_fwd_k##KK(bool bf16, int vec, int unroll, int maxt, const ConvArgs& a, dim3 grid, \
-                                dim3 block, hipStream_t s);                                             \
-    hipError_t launch_bwd_k##KK(bool bf16, int vec, int unroll, int maxt, const ConvArgs& a, dim3 grid, \
-                                dim3 block, size_t shmem, hipStream_t s);
+#define NPLM_DECLARE_K(KK)                                                                               \
+    hipError_t launch_fwd_k##KK(bool bf16, int vec, int unroll, int maxt, const ConvPtrs& p, const Geo& g,   \
+                                dim3 grid, dim3 block, hipStream_t s);                                       \
+    hipError_t launch_bwd_k##KK(bool bf16, int vec, int unroll, int maxt, bool wdx, bool wdw,                \
+                                const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block, size_t shmem,        \
+                                hipStream_t s);
+// Which LDS kernel shape to launch (all are template parameters of the kernels).
+struct LdsShapeSel {
+    bool bf16;
+    int vec, rw, nrg, ncw, nwl;
+};
+#define NPLM_DECLARE_LDS_K(KK)                                                                            \
+    hipError_t launch_fwd_lds_k##KK(const LdsShapeSel& sh, const ConvPtrs& p, const LdsGeo& g, dim3 grid, \
+                                    hipStream_t s);                                                       \
+    hipError_t launch_bwd_lds_k##KK(const LdsShapeSel& sh, bool wdx, bool wdw, const ConvPtrs& p,         \
+                                    const LdsGeo& g, dim3 grid, hipStream_t s);
+NPLM_DECLARE_LDS_K(3)
+NPLM_DECLARE_LDS_K(5)
+NPLM_DECLARE_LDS_K(7)
+NPLM_DECLARE_LDS_K(9)
+#undef NPLM_DECLARE_LDS_K
 NPLM_DECLARE_K(3)
 NPLM_DECLARE_K(5)
 NPLM_DECLARE_K(7)
@@ -74,9 +114,17 @@ constexpr int max_vec(bool bwd, bool bf16, int K) {
     return bwd ? 4 : 8;
 }
 constexpr int default_unroll(bool bwd, int K, int vec) {
-    (void)bwd;
     if (K >= 15) return 4;
+    if (bwd) return vec >= 4 ? 4 : 8;
     return vec >= 8 ? 4 : 8;
+}
+// LDS-staged kernels are built for K <= 9.
+constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+// Default shape: 4 wave-columns of 64 lanes x 8 bytes = 2 KiB of a row per block, 2 row groups,
+// 4 loader waves; 16-row tiles forward, 12-row tiles backward (x and dy tiles, double buffered, must
+// fit 160 KiB of LDS).
+constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16) {
+    return LdsShapeSel{bf16, bf16 ? 4 : 2, bwd ? 6 : 8, 2, 4, 4};
 }
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)K; (void)vec;

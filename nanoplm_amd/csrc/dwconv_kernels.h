@@ -27,17 +27,11 @@
 
 namespace nplm {
 
-struct ConvArgs {
-    const void* x;         // fwd: x          bwd: x
-    const void* dy;        // fwd: unused     bwd: dy
-    const int32_t* cu;     // [S+1]
-    const void* w;         // [C,K] f32 or bf16
-    const void* b;         // fwd: [C] or null
-    void* out;             // fwd: y          bwd: dx (may be null)
-    float* partial;        // bwd: [nbt][K+1][C] fp32 (may be null -> no dw/db)
-    int32_t T, C, S, K;
+// Sizes and launch geometry (everything that is not a pointer). Pointers are passed as separate
+// __restrict__ kernel arguments so that cu is read through the scalar data path.
+struct Geo {
+    int32_t T, C, S;
     int32_t w_bf16;
-    // geometry
     int32_t R;             // rows per tile (multiple of U)
     int32_t ntiles;        // ceil(T / R)
     int32_t ncols;         // C / VEC
@@ -50,28 +44,28 @@ struct ConvArgs {
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
 // blockIdx -> (column-block, token-block). Hardware deals consecutive workgroups round-robin to the
-// 8 XCDs; with xcd_remap, workgroups on one XCD get consecutive logical ids, so tiles that share
-// halo rows meet in the same L2.
-__device__ __forceinline__ void block_coords(const ConvArgs& a, int& cb, int& tb) {
+// 8 XCDs; with xcd_remap, workgroups on one XCD get consecutive logical ids (measured slower on
+// MI355X than the plain order, which keeps all XCDs inside one window of rows; kept as an option).
+__device__ __forceinline__ void block_coords(const Geo& g, int& cb, int& tb) {
     int b = (int)blockIdx.x;
-    if (a.xcd_remap) {
+    if (g.xcd_remap) {
         const int per = (int)(gridDim.x >> 3);
         b = (b & 7) * per + (b >> 3);
     }
-    cb = b % a.ncb;
-    tb = b / a.ncb;
+    cb = b % g.ncb;
+    tb = b / g.ncb;
 }
 
 template <int VEC, int K>
-__device__ __forceinline__ void load_weights(const ConvArgs& a, int c0, float (&wr)[VEC][K]) {
-    if (a.w_bf16) {
-        const uint16_t* wp = reinterpret_cast<const uint16_t*>(a.w) + (size_t)c0 * K;
+__device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_bf16, int c0, float (&wr)[VEC][K]) {
+    if (w_bf16) {
+        const uint16_t* wp = reinterpret_cast<const uint16_t*>(w) + (size_t)c0 * K;
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
 #pragma unroll
             for (int k = 0; k < K; ++k) wr[v][k] = bf16_to_f32(wp[v * K + k]);
     } else {
-        const float* wp = reinterpret_cast<const float*>(a.w) + (size_t)c0 * K;
+        const float* wp = reinterpret_cast<const float*>(w) + (size_t)c0 * K;
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
 #pragma unroll
@@ -81,118 +75,146 @@ __device__ __forceinline__ void load_weights(const ConvArgs& a, int c0, float (&
 
 __device__ __forceinline__ int clamp_row(int r, int T) { return r < 0 ? 0 : (r >= T ? T - 1 : r); }
 
+// Window storage. The K-1+U rows a chunk needs live in a ring of RING row slots; chunk number i of
+// a tile starts at slot (i mod NPH) * U. When NPH * U >= K-1+U for some NPH <= 3 the chunk loop is
+// unrolled NPH times and every slot index is a compile-time constant: no register moves at all.
+// Otherwise (large K) NPH = 1 and the last K-1 rows are moved down after every chunk.
+template <int K, int U> struct Ring {
+    static constexpr int NEED = K - 1 + U;
+    static constexpr int N3 = 1 + (K - 1 + U - 1) / U;          // phases so that (N3-1)*U >= K-1
+    static constexpr bool ROTATE = (K > 1) && (N3 <= 3);
+    static constexpr int NPH = ROTATE ? N3 : 1;
+    static constexpr int RING = ROTATE ? N3 * U : NEED;
+    static constexpr int slot(int ph, int j) { return (ph * U + j) % RING; }
+};
+
 // =============================================================================================
 // Forward
 // =============================================================================================
 template <bool BF16, int K, int VEC, int U, int MAXT>
-__global__ void __launch_bounds__(MAXT) dwconv_fwd_kernel(const ConvArgs a) {
+__global__ void __launch_bounds__(MAXT)
+dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
+                  const void* __restrict__ b, void* __restrict__ y, const Geo g) {
     constexpr int P = (K - 1) / 2;
     constexpr int E = BF16 ? 2 : 4;
     using Row = RowVec<BF16, VEC>;
+    using RG = Ring<K, U>;
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
     int cb, tb;
-    block_coords(a, cb, tb);
-    const int wc = cb * a.bw + (wv % a.bw);
-    const int tslot = tb * a.bt + (wv / a.bw);
-    const int ntslots = a.nbt * a.bt;
-    if (wc >= a.nwc) return;
+    block_coords(g, cb, tb);
+    const int wc = cb * g.bw + (wv % g.bw);
+    const int tslot = tb * g.bt + (wv / g.bw);
+    const int ntslots = g.nbt * g.bt;
+    if (wc >= g.nwc) return;
 
     const int col = wc * 64 + lane;
-    const bool active = col < a.ncols;
-    const int c0 = (active ? col : a.ncols - 1) * VEC;   // clamped: loads stay in bounds, stores are guarded
-    const uint32_t lane_off = (uint32_t)c0 * E;
-    const size_t row_bytes = (size_t)a.C * E;
-    const int T = a.T, S = a.S, R = a.R;
-    const int32_t* __restrict__ cu = a.cu;
-    const char* __restrict__ xb = reinterpret_cast<const char*>(a.x);
-    char* __restrict__ yb = reinterpret_cast<char*>(a.out);
+    const bool active = col < g.ncols;
+    const int c0 = (active ? col : g.ncols - 1) * VEC;   // clamped: loads stay in bounds, stores are guarded
+    const int lane_off = c0 * E;
+    const size_t row_bytes = (size_t)g.C * E;
+    const int rowb = (int)row_bytes;
+    const int T = g.T, S = g.S, R = g.R;
 
     float wr[VEC][K];
-    load_weights<VEC, K>(a, c0, wr);
+    load_weights<VEC, K>(w, g.w_bf16, c0, wr);
     float bias[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
-    if (a.b) {
+    if (b) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
-            bias[v] = a.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(a.b)[c0 + v])
-                               : reinterpret_cast<const float*>(a.b)[c0 + v];
+            bias[v] = g.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
+                               : reinterpret_cast<const float*>(b)[c0 + v];
     }
 
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
 
-    for (int tile = tslot; tile < a.ntiles; tile += ntslots) {
+    for (int tile = tslot; tile < g.ntiles; tile += ntslots) {
         const int t0 = tile * R;
         const int t1 = (t0 + R < T) ? t0 + R : T;
-        sc.locate(cu, S, T, t0, sc.seq);
+        const int rb = (t0 - P > 0) ? t0 - P : 0;            // first row the descriptors cover
+        const rsrc_t rx = rows_rsrc(x, rb, T, row_bytes);
+        const rsrc_t ry = rows_rsrc(y, t0, T, row_bytes);
 
-        float win[K - 1 + U][VEC];   // win[j] = row (tc - P + j)
+        float win[RG::RING][VEC];   // slot(ph, j) holds row tc - P + j
 #pragma unroll
         for (int j = 0; j < K - 1; ++j) {
             Row r;
-            r.load(xb + (size_t)clamp_row(t0 - P + j, T) * row_bytes + lane_off);
-            r.to_f32(win[j]);
+            r.bload(rx, lane_off, (clamp_row(t0 - P + j, T) - rb) * rowb);
+            r.to_f32(win[RG::slot(0, j)]);
         }
         Row nxt[U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) nxt[u].load(xb + (size_t)clamp_row(t0 + P + u, T) * row_bytes + lane_off);
+        for (int u = 0; u < U; ++u) nxt[u].bload(rx, lane_off, (clamp_row(t0 + P + u, T) - rb) * rowb);
+        sc.locate(cu, S, T, t0, sc.seq);
 
-        for (int tc = t0; tc < t1; tc += U) {
+        for (int tc = t0; tc < t1;) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) nxt[u].to_f32(win[K - 1 + u]);
-            if (tc + U < t1) {
+            for (int ph = 0; ph < RG::NPH; ++ph) {
+                if (tc < t1) {
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    nxt[u].load(xb + (size_t)clamp_row(tc + U + P + u, T) * row_bytes + lane_off);
-            }
-            sc.advance(cu, S, T, tc);
-            if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
-                // whole footprint inside one sequence
+                    for (int u = 0; u < U; ++u) nxt[u].to_f32(win[RG::slot(ph, K - 1 + u)]);
+                    if (tc + U < t1) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    float acc[VEC];
+                        for (int u = 0; u < U; ++u)
+                            nxt[u].bload(rx, lane_off, (clamp_row(tc + U + P + u, T) - rb) * rowb);
+                    }
+                    sc.advance(cu, S, T, tc);
+                    Row o[U];
+                    if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
+                        // whole footprint inside one sequence
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+                        for (int u = 0; u < U; ++u) {
+                            float acc[VEC];
 #pragma unroll
-                    for (int k = 0; k < K; ++k)
+                            for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wr[v][k], win[u + k][v], acc[v]);
-                    Row o;
-                    o.from_f32(acc);
-                    if (active) o.store(yb + (size_t)(tc + u) * row_bytes + lane_off);
-                }
-            } else {
+                            for (int k = 0; k < K; ++k)
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int t = tc + u;
-                    if (t < t1) {
-                        sc.advance(cu, S, T, t);
-                        float acc[VEC];
+                                for (int v = 0; v < VEC; ++v)
+                                    acc[v] = __builtin_fmaf(wr[v][k], win[RG::slot(ph, u + k)][v], acc[v]);
+                            o[u].from_f32(acc);
+                        }
+                        if (active) {
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+                            for (int u = 0; u < U; ++u) o[u].bstore(ry, lane_off, (tc + u - t0) * rowb);
+                        }
+                    } else {
 #pragma unroll
-                        for (int k = 0; k < K; ++k) {
-                            const int j = t + k - P;
-                            const bool ok = (j >= sc.cs) && (j < sc.ce);
+                        for (int u = 0; u < U; ++u) {
+                            const int t = tc + u;
+                            if (t < t1) {
+                                sc.advance(cu, S, T, t);
+                                float acc[VEC];
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) {
-                                const float xv = ok ? win[u + k][v] : 0.f;
-                                acc[v] = __builtin_fmaf(wr[v][k], xv, acc[v]);
+                                for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+#pragma unroll
+                                for (int k = 0; k < K; ++k) {
+                                    const int j = t + k - P;
+                                    const bool ok = (j >= sc.cs) && (j < sc.ce);
+#pragma unroll
+                                    for (int v = 0; v < VEC; ++v) {
+                                        const float xv = ok ? win[RG::slot(ph, u + k)][v] : 0.f;
+                                        acc[v] = __builtin_fmaf(wr[v][k], xv, acc[v]);
+                                    }
+                                }
+                                o[u].from_f32(acc);
+                                if (active) o[u].bstore(ry, lane_off, (t - t0) * rowb);
                             }
                         }
-                        Row o;
-                        o.from_f32(acc);
-                        if (active) o.store(yb + (size_t)t * row_bytes + lane_off);
                     }
+                    if constexpr (!RG::ROTATE) {
+#pragma unroll
+                        for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) win[j][v] = win[j + U][v];
+                    }
+                    tc += U;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < K - 1; ++j)
-#pragma unroll
-                for (int v = 0; v < VEC; ++v) win[j][v] = win[j + U][v];
         }
     }
 }
@@ -206,39 +228,38 @@ __global__ void __launch_bounds__(MAXT) dwconv_fwd_kernel(const ConvArgs a) {
 // Each wave keeps dw/db for its VEC channels in registers across all its tiles. At the end the bt
 // waves of a block that share a wave-column are summed through LDS in fixed order (token slot
 // 0,1,2,...), and the block writes one slab partial[tb][k][c]. No atomics.
-template <bool BF16, int K, int VEC, int U, int MAXT>
-__global__ void __launch_bounds__(MAXT) dwconv_bwd_kernel(const ConvArgs a) {
+// WDX / WDW select the outputs at compile time (dx only, dw/db only, or both).
+template <bool BF16, int K, int VEC, int U, int MAXT, bool WDX, bool WDW>
+__global__ void __launch_bounds__(MAXT)
+dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
+                  const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const Geo g) {
     constexpr int P = (K - 1) / 2;
     constexpr int E = BF16 ? 2 : 4;
     using Row = RowVec<BF16, VEC>;
+    using RG = Ring<K, U>;
     extern __shared__ float red[];   // [nwaves][VEC][64]
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
     int cb, tb;
-    block_coords(a, cb, tb);
-    const int wcl = wv % a.bw;
-    const int tl = wv / a.bw;
-    const int wc = cb * a.bw + wcl;
-    const int tslot = tb * a.bt + tl;
-    const int ntslots = a.nbt * a.bt;
-    const bool wave_on = wc < a.nwc;   // idle waves still take part in the barriers below
+    block_coords(g, cb, tb);
+    const int wcl = wv % g.bw;
+    const int tl = wv / g.bw;
+    const int wc = cb * g.bw + wcl;
+    const int tslot = tb * g.bt + tl;
+    const int ntslots = g.nbt * g.bt;
+    const bool wave_on = wc < g.nwc;   // idle waves still take part in the barriers below
 
     const int col = wc * 64 + lane;
-    const bool active = wave_on && col < a.ncols;
-    const int c0 = (active ? col : a.ncols - 1) * VEC;
-    const uint32_t lane_off = (uint32_t)c0 * E;
-    const size_t row_bytes = (size_t)a.C * E;
-    const int T = a.T, S = a.S, R = a.R;
-    const int32_t* __restrict__ cu = a.cu;
-    const char* __restrict__ xb = reinterpret_cast<const char*>(a.x);
-    const char* __restrict__ gb = reinterpret_cast<const char*>(a.dy);
-    char* __restrict__ ob = reinterpret_cast<char*>(a.out);
-    const bool want_dx = ob != nullptr;
-    const bool want_dw = a.partial != nullptr;
+    const bool active = wave_on && col < g.ncols;
+    const int c0 = (active ? col : g.ncols - 1) * VEC;
+    const int lane_off = c0 * E;
+    const size_t row_bytes = (size_t)g.C * E;
+    const int rowb = (int)row_bytes;
+    const int T = g.T, S = g.S, R = g.R;
 
     float wr[VEC][K];
-    load_weights<VEC, K>(a, c0, wr);
+    if constexpr (WDX) load_weights<VEC, K>(w, g.w_bf16, c0, wr);
     float dwa[VEC][K];
     float dba[VEC];
 #pragma unroll
@@ -252,104 +273,138 @@ __global__ void __launch_bounds__(MAXT) dwconv_bwd_kernel(const ConvArgs a) {
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
 
     if (wave_on) {
-        for (int tile = tslot; tile < a.ntiles; tile += ntslots) {
+        for (int tile = tslot; tile < g.ntiles; tile += ntslots) {
             const int t0 = tile * R;
             const int t1 = (t0 + R < T) ? t0 + R : T;
-            sc.locate(cu, S, T, t0, sc.seq);
+            const int rb = (t0 - P > 0) ? t0 - P : 0;
+            const rsrc_t rx = rows_rsrc(x, rb, T, row_bytes);
+            const rsrc_t rg = rows_rsrc(dy, rb, T, row_bytes);
+            const rsrc_t ro = rows_rsrc(dx, t0, T, row_bytes);
 
-            float xw[K - 1 + U][VEC];   // x  rows tc-P .. tc+U-1+P
-            float gw[K - 1 + U][VEC];   // dy rows, same range
+            float xw[WDW ? RG::RING : 1][VEC];   // x  rows tc-P .. tc+U-1+P
+            float gw[RG::RING][VEC];             // dy rows, same range
 #pragma unroll
             for (int j = 0; j < K - 1; ++j) {
-                const size_t off = (size_t)clamp_row(t0 - P + j, T) * row_bytes + lane_off;
+                const int so = (clamp_row(t0 - P + j, T) - rb) * rowb;
                 Row r;
-                r.load(xb + off); r.to_f32(xw[j]);
-                r.load(gb + off); r.to_f32(gw[j]);
+                if constexpr (WDW) { r.bload(rx, lane_off, so); r.to_f32(xw[RG::slot(0, j)]); }
+                r.bload(rg, lane_off, so); r.to_f32(gw[RG::slot(0, j)]);
             }
-            Row nx[U], ng[U];
+            Row nx[WDW ? U : 1], ng[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const size_t off = (size_t)clamp_row(t0 + P + u, T) * row_bytes + lane_off;
-                nx[u].load(xb + off);
-                ng[u].load(gb + off);
+                const int so = (clamp_row(t0 + P + u, T) - rb) * rowb;
+                if constexpr (WDW) nx[u].bload(rx, lane_off, so);
+                ng[u].bload(rg, lane_off, so);
             }
+            sc.locate(cu, S, T, t0, sc.seq);
 
-            for (int tc = t0; tc < t1; tc += U) {
+            for (int tc = t0; tc < t1;) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) { nx[u].to_f32(xw[K - 1 + u]); ng[u].to_f32(gw[K - 1 + u]); }
-                if (tc + U < t1) {
+                for (int ph = 0; ph < RG::NPH; ++ph) {
+                    if (tc < t1) {
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        const size_t off = (size_t)clamp_row(tc + U + P + u, T) * row_bytes + lane_off;
-                        nx[u].load(xb + off);
-                        ng[u].load(gb + off);
-                    }
-                }
-                sc.advance(cu, S, T, tc);
-                if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
-#pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        float g[VEC];
-#pragma unroll
-                        for (int v = 0; v < VEC; ++v) { g[v] = gw[u + P][v]; dba[v] += g[v]; }
-#pragma unroll
-                        for (int k = 0; k < K; ++k)
-#pragma unroll
-                            for (int v = 0; v < VEC; ++v) dwa[v][k] = __builtin_fmaf(g[v], xw[u + k][v], dwa[v][k]);
-                        if (want_dx) {
-                            float acc[VEC];
-#pragma unroll
-                            for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
-#pragma unroll
-                            for (int m = 0; m < K; ++m)
-#pragma unroll
-                                for (int v = 0; v < VEC; ++v) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gw[u + m][v], acc[v]);
-                            Row o;
-                            o.from_f32(acc);
-                            if (active) o.store(ob + (size_t)(tc + u) * row_bytes + lane_off);
+                        for (int u = 0; u < U; ++u) {
+                            if constexpr (WDW) nx[u].to_f32(xw[RG::slot(ph, K - 1 + u)]);
+                            ng[u].to_f32(gw[RG::slot(ph, K - 1 + u)]);
                         }
-                    }
-                } else {
+                        if (tc + U < t1) {
 #pragma unroll
-                    for (int u = 0; u < U; ++u) {
-                        const int t = tc + u;
-                        if (t < t1) {
-                            sc.advance(cu, S, T, t);
-                            float g[VEC], acc[VEC];
+                            for (int u = 0; u < U; ++u) {
+                                const int so = (clamp_row(tc + U + P + u, T) - rb) * rowb;
+                                if constexpr (WDW) nx[u].bload(rx, lane_off, so);
+                                ng[u].bload(rg, lane_off, so);
+                            }
+                        }
+                        sc.advance(cu, S, T, tc);
+                        Row o[WDX ? U : 1];
+                        if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) { g[v] = gw[u + P][v]; dba[v] += g[v]; acc[v] = 0.f; }
+                            for (int u = 0; u < U; ++u) {
+                                if constexpr (WDW) {
+                                    float gc[VEC];
 #pragma unroll
-                            for (int m = 0; m < K; ++m) {
-                                const int j = t + m - P;
-                                const bool ok = (j >= sc.cs) && (j < sc.ce);
+                                    for (int v = 0; v < VEC; ++v) { gc[v] = gw[RG::slot(ph, u + P)][v]; dba[v] += gc[v]; }
 #pragma unroll
-                                for (int v = 0; v < VEC; ++v) {
-                                    const float xv = ok ? xw[u + m][v] : 0.f;
-                                    const float gv = ok ? gw[u + m][v] : 0.f;
-                                    dwa[v][m] = __builtin_fmaf(g[v], xv, dwa[v][m]);
-                                    acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
+                                    for (int k = 0; k < K; ++k)
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v)
+                                            dwa[v][k] = __builtin_fmaf(gc[v], xw[RG::slot(ph, u + k)][v], dwa[v][k]);
+                                }
+                                if constexpr (WDX) {
+                                    float acc[VEC];
+#pragma unroll
+                                    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+#pragma unroll
+                                    for (int m = 0; m < K; ++m)
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v)
+                                            acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gw[RG::slot(ph, u + m)][v], acc[v]);
+                                    o[u].from_f32(acc);
                                 }
                             }
-                            if (want_dx) {
-                                Row o;
-                                o.from_f32(acc);
-                                if (active) o.store(ob + (size_t)t * row_bytes + lane_off);
+                            if constexpr (WDX) {
+                                if (active) {
+#pragma unroll
+                                    for (int u = 0; u < U; ++u) o[u].bstore(ro, lane_off, (tc + u - t0) * rowb);
+                                }
+                            }
+                        } else {
+#pragma unroll
+                            for (int u = 0; u < U; ++u) {
+                                const int t = tc + u;
+                                if (t < t1) {
+                                    sc.advance(cu, S, T, t);
+                                    float gc[VEC], acc[VEC];
+#pragma unroll
+                                    for (int v = 0; v < VEC; ++v) {
+                                        gc[v] = gw[RG::slot(ph, u + P)][v];
+                                        if constexpr (WDW) dba[v] += gc[v];
+                                        acc[v] = 0.f;
+                                    }
+#pragma unroll
+                                    for (int m = 0; m < K; ++m) {
+                                        const int j = t + m - P;
+                                        const bool ok = (j >= sc.cs) && (j < sc.ce);
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v) {
+                                            if constexpr (WDW) {
+                                                const float xv = ok ? xw[RG::slot(ph, u + m)][v] : 0.f;
+                                                dwa[v][m] = __builtin_fmaf(gc[v], xv, dwa[v][m]);
+                                            }
+                                            if constexpr (WDX) {
+                                                const float gv = ok ? gw[RG::slot(ph, u + m)][v] : 0.f;
+                                                acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
+                                            }
+                                        }
+                                    }
+                                    if constexpr (WDX) {
+                                        o[u].from_f32(acc);
+                                        if (active) o[u].bstore(ro, lane_off, (t - t0) * rowb);
+                                    }
+                                }
                             }
                         }
+                        if constexpr (!RG::ROTATE) {
+#pragma unroll
+                            for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    if constexpr (WDW) xw[j][v] = xw[j + U][v];
+                                    gw[j][v] = gw[j + U][v];
+                                }
+                        }
+                        tc += U;
                     }
                 }
-#pragma unroll
-                for (int j = 0; j < K - 1; ++j)
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) { xw[j][v] = xw[j + U][v]; gw[j][v] = gw[j + U][v]; }
             }
         }
     }
 
-    if (!want_dw) return;   // uniform over the grid
+    if constexpr (!WDW) return;
 
     // ---- block-level pass: sum the bt token slots of each wave-column, slot order 0,1,2,... ----
-    float* slab = a.partial + (size_t)tb * (K + 1) * a.C;
+    float* slab = partial + (size_t)tb * (K + 1) * g.C;
 #pragma unroll
     for (int kk = 0; kk <= K; ++kk) {
         float val[VEC];
@@ -361,13 +416,13 @@ __global__ void __launch_bounds__(MAXT) dwconv_bwd_kernel(const ConvArgs a) {
         }
         __syncthreads();
         if (tl == 0) {
-            for (int j = 1; j < a.bt; ++j) {
-                const int ow = j * a.bw + wcl;
+            for (int j = 1; j < g.bt; ++j) {
+                const int ow = j * g.bw + wcl;
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
             }
             if (active) {
-                float* dst = slab + (size_t)kk * a.C + c0;
+                float* dst = slab + (size_t)kk * g.C + c0;
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) dst[v] = val[v];
             }

@@ -1,0 +1,434 @@
+// LDS-staged, software-pipelined kernels of the varlen depthwise conv (gfx950, wave64), for small
+// kernel sizes.
+//
+// A block owns tiles of R = RW*NRG consecutive token rows x one column block of NCW*64*VEC channels
+// (2 KiB of every row at the default sizes). Its waves have two roles:
+//
+//   loader waves (NWL)   issue direct global->LDS loads (buffer_load ... lds, 16 B per lane,
+//                        consecutive lanes consecutive addresses) for the NEXT tile and its K-1 halo
+//                        rows, then wait for them. Every row of a tile is one contiguous run in HBM
+//                        and is fetched once per block; no vector registers are involved.
+//   compute waves        (NCW wave-columns x NRG row groups) work on the CURRENT tile out of LDS:
+//                        each reads its RW+K-1 rows once, scatters every row into the RW accumulators
+//                        it contributes to, and stores RW output rows.
+//
+// The two tiles live in two LDS buffers; one workgroup barrier per tile hands the freshly loaded
+// buffer to the compute waves and the consumed one back to the loaders, so HBM traffic and
+// arithmetic overlap inside one block. Blocks walk tiles grid-stride (tile, tile + nbt, ...): all
+// resident blocks together sweep one compact window of rows, the access pattern HBM serves fastest,
+// and the halo rows a block re-reads were fetched moments earlier by its neighbour.
+//
+// Backward: x and dy tiles are staged the same way; dx is written per tile, dw/db stay in registers
+// across all tiles of the block and are combined as in the sliding-window kernels (row groups summed
+// through LDS in fixed order, one slab per token-block, then dwconv_finalize_kernel). No atomics.
+//
+// Every wave of a block executes exactly the same sequence of barriers: the trip counts depend only
+// on blockIdx and the launch geometry.
+//
+// No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); tensor contract:
+// modeling.py:339,421-439 and collator.py:322-325,405-458.
+#pragma once
+#include "dwconv_kernels.h"
+
+namespace nplm {
+
+struct LdsGeo {
+    int32_t T, C, S;
+    int32_t w_bf16;
+    int32_t ntiles;     // ceil(T / R)
+    int32_t ncb, nbt;   // grid = ncb column blocks x nbt token blocks (nbt <= ntiles)
+};
+
+typedef __attribute__((address_space(3))) void lds_void;
+
+// s_waitcnt vmcnt(0) (expcnt / lgkmcnt untouched), gfx9 encoding.
+__device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// Compile-time shape of one kernel variant.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL>
+struct LdsShape {
+    static constexpr int E = BF16 ? 2 : 4;
+    static constexpr int P = (K - 1) / 2;
+    static constexpr int NWC = NCW * NRG;               // compute waves
+    static constexpr int NT = (NWC + NWL) * 64;         // threads per block
+    static constexpr int R = RW * NRG;                  // output rows per tile
+    static constexpr int NROWS = R + K - 1;             // staged rows per tile
+    static constexpr int CB_BYTES = NCW * 64 * VEC * E; // bytes of a row in one column block
+    static constexpr int CB_CH = NCW * 64 * VEC;        // channels in one column block
+    static constexpr int NPIECE = CB_BYTES / 1024;      // 1 KiB direct loads per staged row
+    static constexpr int TILE_BYTES = NROWS * CB_BYTES;
+    static_assert(CB_BYTES % 1024 == 0, "a column block must be a whole number of 1 KiB wave loads");
+    static_assert((NPIECE & (NPIECE - 1)) == 0, "pieces per row must be a power of two");
+    static_assert(NROWS * CB_BYTES <= 65536, "ds_read immediate offsets are 16 bit");
+};
+
+// Loader: stage rows t0-P .. t0-P+NROWS-1 (clamped to [0,T)) x this block's column block of `src`
+// into `dst` (row pitch CB_BYTES). (row, piece) pairs are dealt round-robin to the loader waves.
+template <typename SH>
+__device__ __forceinline__ void stage_tile(const void* __restrict__ src, char* dst, int t0, int T, size_t row_bytes,
+                                           int col_byte0, int valid_bytes, int lw, int nlw, int lane) {
+    const int rb = (t0 - SH::P > 0) ? t0 - SH::P : 0;
+    const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
+    const int rowb = (int)row_bytes;
+    const int voff = lane * 16;
+    for (int pair = lw; pair < SH::NROWS * SH::NPIECE; pair += nlw) {
+        const int j = pair / SH::NPIECE;
+        const int p = pair % SH::NPIECE;
+        const int so = (clamp_row(t0 - SH::P + j, T) - rb) * rowb + col_byte0 + p * 1024;
+        char* d = dst + j * SH::CB_BYTES + p * 1024;
+        if (p * 1024 + voff < valid_bytes)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, voff, so, 0, 0);
+    }
+}
+
+template <bool BF16, int VEC>
+__device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
+    RowVec<BF16, VEC> r;
+    r.load(p);
+    r.to_f32(f);
+}
+
+// Per-output-row tap limits of a wave's RW rows: tap row g is valid for output u iff lo[u] <= g < hi[u].
+template <int RW>
+struct WaveBounds {
+    bool interior;   // every tap of every row of the wave lies inside one sequence
+    int lo[RW], hi[RW];
+};
+
+template <int RW, int P>
+__device__ __forceinline__ void wave_bounds(SeqCursor& sc, const int32_t* __restrict__ cu, int S, int T, int tf,
+                                            WaveBounds<RW>& wb) {
+    // tf = first output row of the wave (tf < T)
+    sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
+    const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
+    wb.interior = (tf - P >= sc.cs) && (tl + P < sc.ce);
+    if (!wb.interior) {
+#pragma unroll
+        for (int u = 0; u < RW; ++u) {
+            const int t = tf + u;
+            if (t < T) sc.advance(cu, S, T, t);
+            wb.lo[u] = sc.cs;
+            wb.hi[u] = sc.ce;
+        }
+    }
+}
+
+// =============================================================================================
+// Forward
+// =============================================================================================
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL>
+__global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
+dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
+                      const void* __restrict__ b, void* __restrict__ y, const LdsGeo g) {
+    using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
+    constexpr int P = SH::P, E = SH::E, R = SH::R;
+    using Row = RowVec<BF16, VEC>;
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x TILE_BYTES
+
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    const bool is_loader = wv >= SH::NWC;
+    const int cb = (int)blockIdx.x % g.ncb;
+    const int tb = (int)blockIdx.x / g.ncb;
+    const int T = g.T, S = g.S, C = g.C;
+    const size_t row_bytes = (size_t)C * E;
+    const int rowb = (int)row_bytes;
+    const int col_byte0 = cb * SH::CB_BYTES;
+    const int valid_bytes = (rowb - col_byte0 < SH::CB_BYTES) ? rowb - col_byte0 : SH::CB_BYTES;
+    const int ntl = (g.ntiles - tb + g.nbt - 1) / g.nbt;   // tiles of this block (>= 1), same for all waves
+
+    // compute-wave coordinates (meaningless but harmless for loader waves)
+    const int wc = wv % NCW;
+    const int rg = (wv / NCW) % NRG;
+    const int cw = valid_bytes / E;                                  // channels in this column block
+    const int lcol = (wc * 64 + lane) * VEC;
+    const bool active = !is_loader && lcol < cw;
+    const int lc0 = (lcol < cw) ? lcol : cw - VEC;
+    const int c0 = cb * SH::CB_CH + lc0;
+    const int out_voff = c0 * E;
+
+    float wr[VEC][K];
+    float bias[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
+    if (is_loader) {
+        stage_tile<SH>(x, lds_raw, tb * R, T, row_bytes, col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
+        wait_vmem_all();
+    } else {
+        load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+        if (b) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v)
+                bias[v] = g.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
+                                   : reinterpret_cast<const float*>(b)[c0 + v];
+        }
+    }
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    __syncthreads();
+
+    for (int it = 0; it < ntl; ++it) {
+        const int t0 = (tb + it * g.nbt) * R;
+        char* cur = lds_raw + (it & 1) * SH::TILE_BYTES;
+        if (is_loader) {
+            if (it + 1 < ntl) {
+                stage_tile<SH>(x, lds_raw + ((it + 1) & 1) * SH::TILE_BYTES, t0 + g.nbt * R, T, row_bytes, col_byte0,
+                               valid_bytes, wv - SH::NWC, NWL, lane);
+                wait_vmem_all();
+            }
+        } else {
+            const int tf = t0 + rg * RW;
+            if (tf < T) {
+                WaveBounds<RW> wb;
+                wave_bounds<RW, P>(sc, cu, S, T, tf, wb);
+                float acc[RW][VEC];
+#pragma unroll
+                for (int u = 0; u < RW; ++u)
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v) acc[u][v] = bias[v];
+                const char* lp = cur + (rg * RW) * SH::CB_BYTES + lc0 * E;
+                if (wb.interior) {
+#pragma unroll
+                    for (int j = 0; j < RW + K - 1; ++j) {
+                        float xr[VEC];
+                        lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) {
+                            if (j - u >= 0 && j - u < K) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) acc[u][v] = __builtin_fmaf(wr[v][j - u], xr[v], acc[u][v]);
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < RW + K - 1; ++j) {
+                        float xr[VEC];
+                        lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+                        const int gr = tf - P + j;
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) {
+                            if (j - u >= 0 && j - u < K) {
+                                const bool ok = (gr >= wb.lo[u]) && (gr < wb.hi[u]);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    const float xv = ok ? xr[v] : 0.f;
+                                    acc[u][v] = __builtin_fmaf(wr[v][j - u], xv, acc[u][v]);
+                                }
+                            }
+                        }
+                    }
+                }
+                const rsrc_t ry = rows_rsrc(y, tf, T, row_bytes);
+                Row o[RW];
+#pragma unroll
+                for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                if (active) {
+#pragma unroll
+                    for (int u = 0; u < RW; ++u)
+                        if (tf + u < T) o[u].bstore(ry, out_voff, u * rowb);
+                }
+            }
+        }
+        __syncthreads();   // next tile is in LDS; this tile's buffer may be overwritten
+    }
+}
+
+// =============================================================================================
+// Backward (fused)
+// =============================================================================================
+// LDS: [2 buffers][x tile, dy tile]; without dw/db (WDW = false) only the dy tiles are staged.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW>
+__global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
+dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
+                      const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
+    using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
+    constexpr int P = SH::P, E = SH::E, R = SH::R;
+    constexpr int NTENS = WDW ? 2 : 1;
+    constexpr int BUF_BYTES = NTENS * SH::TILE_BYTES;
+    using Row = RowVec<BF16, VEC>;
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
+
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    const bool is_loader = wv >= SH::NWC;
+    const int cb = (int)blockIdx.x % g.ncb;
+    const int tb = (int)blockIdx.x / g.ncb;
+    const int T = g.T, S = g.S, C = g.C;
+    const size_t row_bytes = (size_t)C * E;
+    const int rowb = (int)row_bytes;
+    const int col_byte0 = cb * SH::CB_BYTES;
+    const int valid_bytes = (rowb - col_byte0 < SH::CB_BYTES) ? rowb - col_byte0 : SH::CB_BYTES;
+    const int ntl = (g.ntiles - tb + g.nbt - 1) / g.nbt;
+
+    const int wc = wv % NCW;
+    const int rg = (wv / NCW) % NRG;
+    const int cw = valid_bytes / E;
+    const int lcol = (wc * 64 + lane) * VEC;
+    const bool active = !is_loader && lcol < cw;
+    const int lc0 = (lcol < cw) ? lcol : cw - VEC;
+    const int c0 = cb * SH::CB_CH + lc0;
+    const int out_voff = c0 * E;
+    const int lw = wv - SH::NWC;
+
+    // buffer layout: dy tile first, then (if staged) the x tile
+    auto stage_both = [&](char* buf, int t0) {
+        // loader waves split the two tensors between them when there are at least two of them
+        if constexpr (WDW && NWL >= 2) {
+            if (lw & 1) stage_tile<SH>(x, buf + SH::TILE_BYTES, t0, T, row_bytes, col_byte0, valid_bytes, lw >> 1, NWL / 2, lane);
+            else        stage_tile<SH>(dy, buf, t0, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane);
+        } else {
+            stage_tile<SH>(dy, buf, t0, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+            if constexpr (WDW) stage_tile<SH>(x, buf + SH::TILE_BYTES, t0, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+        }
+    };
+
+    float wr[VEC][K];
+    float dwa[VEC][K];
+    float dba[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) {
+        dba[v] = 0.f;
+#pragma unroll
+        for (int k = 0; k < K; ++k) { dwa[v][k] = 0.f; wr[v][k] = 0.f; }
+    }
+    if (is_loader) {
+        stage_both(lds_raw, tb * R);
+        wait_vmem_all();
+    } else {
+        if constexpr (WDX) load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+    }
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    __syncthreads();
+
+    for (int it = 0; it < ntl; ++it) {
+        const int t0 = (tb + it * g.nbt) * R;
+        char* cur = lds_raw + (it & 1) * BUF_BYTES;
+        if (is_loader) {
+            if (it + 1 < ntl) {
+                stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, t0 + g.nbt * R);
+                wait_vmem_all();
+            }
+        } else {
+            const int tf = t0 + rg * RW;
+            if (tf < T) {
+                WaveBounds<RW> wb;
+                wave_bounds<RW, P>(sc, cu, S, T, tf, wb);
+                const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
+                const char* lpg = cur + loff;
+                const char* lpx = cur + SH::TILE_BYTES + loff;
+                // centre dy rows of the wave's outputs (staged row u + P); rows past T contribute nothing
+                float gc[WDW ? RW : 1][VEC];
+                if constexpr (WDW) {
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) {
+                        lds_read_row<BF16, VEC>(lpg + (u + P) * SH::CB_BYTES, gc[u]);
+                        if (tf + u >= T) {
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) gc[u][v] = 0.f;
+                        }
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) dba[v] += gc[u][v];
+                    }
+                }
+                float acc[WDX ? RW : 1][VEC];
+                if constexpr (WDX) {
+#pragma unroll
+                    for (int u = 0; u < RW; ++u)
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) acc[u][v] = 0.f;
+                }
+                if (wb.interior) {
+#pragma unroll
+                    for (int j = 0; j < RW + K - 1; ++j) {
+                        float xr[VEC], gr[VEC];
+                        if constexpr (WDW) lds_read_row<BF16, VEC>(lpx + j * SH::CB_BYTES, xr);
+                        if constexpr (WDX) lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) {
+                            if (j - u >= 0 && j - u < K) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    if constexpr (WDW) dwa[v][j - u] = __builtin_fmaf(gc[u][v], xr[v], dwa[v][j - u]);
+                                    if constexpr (WDX) acc[u][v] = __builtin_fmaf(wr[v][K - 1 - (j - u)], gr[v], acc[u][v]);
+                                }
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < RW + K - 1; ++j) {
+                        float xr[VEC], gr[VEC];
+                        if constexpr (WDW) lds_read_row<BF16, VEC>(lpx + j * SH::CB_BYTES, xr);
+                        if constexpr (WDX) lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        const int grow = tf - P + j;
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) {
+                            if (j - u >= 0 && j - u < K) {
+                                const bool ok = (grow >= wb.lo[u]) && (grow < wb.hi[u]);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    if constexpr (WDW) {
+                                        const float xv = ok ? xr[v] : 0.f;
+                                        dwa[v][j - u] = __builtin_fmaf(gc[u][v], xv, dwa[v][j - u]);
+                                    }
+                                    if constexpr (WDX) {
+                                        const float gv = ok ? gr[v] : 0.f;
+                                        acc[u][v] = __builtin_fmaf(wr[v][K - 1 - (j - u)], gv, acc[u][v]);
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+                if constexpr (WDX) {
+                    const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
+                    Row o[RW];
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                    if (active) {
+#pragma unroll
+                        for (int u = 0; u < RW; ++u)
+                            if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    if constexpr (!WDW) return;
+
+    // ---- block-level pass: sum the NRG row groups of each wave-column, group order 0,1,2,... ----
+    // (the tiles are dead after the last barrier above; loader waves only keep the barriers company)
+    float* red = reinterpret_cast<float*>(lds_raw);   // [NWC][VEC][64]
+    float* slab = partial + (size_t)tb * (K + 1) * C;
+#pragma unroll
+    for (int kk = 0; kk <= K; ++kk) {
+        float val[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) val[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : dba[v];
+        if (!is_loader && rg > 0) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) red[(wv * VEC + v) * 64 + lane] = val[v];
+        }
+        __syncthreads();
+        if (!is_loader && rg == 0) {
+#pragma unroll
+            for (int j = 1; j < NRG; ++j) {
+                const int ow = j * NCW + wc;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
+            }
+            if (active) {
+                float* dst = slab + (size_t)kk * C + c0;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) dst[v] = val[v];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace nplm

@@ -226,20 +226,40 @@ def test_malformed_cu_seqlens_cannot_fault():
 
 
 # ---- launch geometry --------------------------------------------------------------------------------
-@pytest.mark.parametrize("tile_rows,bt,nbt,remap", [(8, 1, 1, 2), (16, 2, 3, 2), (64, 4, 8, 1), (128, 2, 16, 1),
-                                                    (40, 1, 64, 1), (256, 4, 200, 2)])
-def test_results_do_not_depend_on_launch_geometry(tile_rows, bt, nbt, remap):
-    """y and dx are bit-identical for any tiling; dw/db differ only by summation order."""
+SLIDING = [dict(algo=1, tile_rows=8, bt=1, nbt=1), dict(algo=1, tile_rows=16, bt=2, nbt=3),
+           dict(algo=1, tile_rows=64, bt=4, nbt=8, xcd_remap=1), dict(algo=1, tile_rows=128, bt=2, nbt=16, xcd_remap=1),
+           dict(algo=1, tile_rows=40, bt=1, nbt=64), dict(algo=1, tile_rows=256, bt=4, nbt=200), dict(algo=1)]
+LDS = [dict(algo=2), dict(algo=2, nbt=1), dict(algo=2, nbt=7), dict(algo=2, nbt=100000), dict(algo=2, nbt=33)]
+
+
+@pytest.mark.parametrize("tune", SLIDING + LDS, ids=lambda d: "-".join(f"{k}{v}" for k, v in d.items()))
+def test_results_do_not_depend_on_launch_geometry(tune):
+    """y and dx are bit-identical for either kernel family and any tiling; dw/db differ only by
+    summation order."""
     wl, y64, dx64, dw64, db64 = workload_with_oracle(5, 9000, 1024)
     d = wl.to(DEV)
     y0, dx0, dw0, db0 = _run_all(d)
-    tf = _lib.Tuning(tile_rows=tile_rows, bt=bt, nbt=nbt, xcd_remap=remap)
+    tf = _lib.Tuning(**tune)
     y = npa.varlen_dwconv_fwd(d.x, d.cu_seqlens, d.weight, d.bias, tuning=tf)
     dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, tuning=tf)
     assert torch.equal(y, y0) and torch.equal(dx, dx0)
     assert_red_close(dw, dw64, "dw")
     assert_red_close(db, db64, "db")
     torch.testing.assert_close(dw, dw0, rtol=1e-5, atol=1e-3)
+
+
+@pytest.mark.parametrize("algo", [1, 2])
+@pytest.mark.parametrize("index,T,C", [(5, 20000, 1024), (2, 9000, 2048), (2, 5000, 520)])
+def test_both_kernel_families_match_the_oracle(algo, index, T, C):
+    wl, y64, dx64, dw64, db64 = workload_with_oracle(index, T, C)
+    d = wl.to(DEV)
+    tf = _lib.Tuning(algo=algo)
+    y = npa.varlen_dwconv_fwd(d.x, d.cu_seqlens, d.weight, d.bias, tuning=tf)
+    dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight, tuning=tf)
+    assert_act_close(y, y64, wl.dtype, "y")
+    assert_act_close(dx, dx64, wl.dtype, "dx")
+    assert_red_close(dw, dw64, "dw")
+    assert_red_close(db, db64, "db")
 
 
 def test_backward_outputs_can_be_requested_separately():
