@@ -31,7 +31,7 @@ class Tuning(ctypes.Structure):
     """Mirror of ``nplm_dwconv_tuning`` (csrc/dwconv_internal.h); 0 keeps the library default."""
 
     _fields_ = [(n, ctypes.c_int32) for n in
-                ("vec", "unroll", "tile_rows", "bw", "bt", "nbt", "xcd_remap", "maxt", "algo", "nwl", "reserved")
+                ("vec", "unroll", "tile_rows", "bw", "bt", "nbt", "xcd_remap", "maxt", "algo", "nwl", "nbuf")
                 ] + [("mid_event", ctypes.c_void_p)]
 
 

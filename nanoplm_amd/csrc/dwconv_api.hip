@@ -67,7 +67,7 @@ int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bi
     p.unroll = tune->unroll > 0 ? tune->unroll : default_unroll(bwd, K, p.vec);
     p.maxt = tune->maxt > 0 ? tune->maxt : default_maxt(bwd, K, p.vec);
     if (p.maxt < 64 || p.maxt > 1024 || p.maxt % 64) return -NPLM_DWCONV_ETUNING;
-    int R = tune->tile_rows > 0 ? tune->tile_rows : (bwd ? 128 : 64);
+    int R = tune->tile_rows > 0 ? tune->tile_rows : (bwd ? 32 : 64);
     if (R > kMaxTileRows || p.unroll > 64) return -NPLM_DWCONV_ETUNING;
     R = ceil_div(R, p.unroll) * p.unroll;
     // row offsets inside a tile are 32-bit byte offsets
@@ -153,7 +153,7 @@ constexpr size_t kLdsBytesPerCU = 160u << 10;
 
 struct LdsPlan {
     LdsShapeSel sh;
-    int R, ntiles, ncb, nbt;
+    int R, ntiles, ncb, nbt, xcd_group;
 };
 
 // Whether the LDS kernels can take this problem at all (16-byte row granularity, built kernel size).
@@ -175,10 +175,11 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     if (tune->bt > 0) p.sh.nrg = tune->bt;
     if (tune->bw > 0) p.sh.ncw = tune->bw;
     if (tune->nwl > 0) p.sh.nwl = tune->nwl;
+    if (tune->nbuf > 0 && !bwd) p.sh.nbuf = tune->nbuf;
     const long long cb_bytes = (long long)p.sh.ncw * 64 * p.sh.vec * E;
     const long long row_bytes = (long long)C * E;
     p.R = p.sh.rw * p.sh.nrg;
-    const size_t shmem = (size_t)(bwd ? 4 : 2) * (p.R + K - 1) * cb_bytes;
+    const size_t shmem = (size_t)p.sh.nbuf * ((size_t)(p.R + K - 1) + (bwd ? p.R : 0)) * cb_bytes;
     if (shmem > kLdsBytesPerCU || cb_bytes % 1024) return -NPLM_DWCONV_ETUNING;
     if ((long long)(p.R + K) * row_bytes + row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
     p.ncb = ceil_div(row_bytes, cb_bytes);
@@ -192,6 +193,11 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
         if (nbt > cap && cap >= 1) nbt = (int)cap;
     }
     p.nbt = nbt;
+    // adjacent tiles share an XCD in runs of G (tune->xcd_remap: 0 = default 8, > 0 = G, < 0 = off)
+    int G = tune->xcd_remap == 0 ? 8 : (tune->xcd_remap > 0 ? tune->xcd_remap : 0);
+    const long long nblocks = (long long)p.ncb * p.nbt;
+    if (G > 0 && !(nblocks % kNumXCD == 0 && (nblocks / kNumXCD) % G == 0 && p.nbt % G == 0)) G = 0;
+    p.xcd_group = G;
     *out = p;
     return 0;
 }
@@ -199,7 +205,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
 LdsGeo make_lds_geo(const LdsPlan& p, long long T, int C, int S, int w_bf16) {
     LdsGeo g{};
     g.T = (int32_t)T; g.C = C; g.S = S; g.w_bf16 = w_bf16;
-    g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt;
+    g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_group = p.xcd_group;
     return g;
 }
 

@@ -24,12 +24,13 @@ typedef struct nplm_dwconv_tuning {
     int32_t maxt;       // launch-bounds class (threads per block the kernel was compiled for)
     int32_t algo;       // 1 = sliding-window (register) kernels, 2 = LDS-staged pipelined kernels
     int32_t nwl;        // LDS kernels: loader waves per block
-    int32_t reserved;
+    int32_t nbuf;       // LDS forward: tile buffers (2 or 3)
     void* mid_event;    // backward: hipEvent_t recorded between the fused kernel and the finalize kernel
 } nplm_dwconv_tuning;
 // For algo 2 the fields mean: vec = channels per lane, unroll = rows per wave (RW), bt = row groups
 // per block (tile rows = RW * bt), bw = wave-columns per block, nwl = loader waves, nbt = token
-// blocks; tile_rows, xcd_remap and maxt are ignored. Only shapes the library was built with exist.
+// blocks, xcd_remap = run length of adjacent tiles that share an XCD (0 = default 8, < 0 = off);
+// tile_rows and maxt are ignored. Only shapes the library was built with exist.
 
 // Same contracts as nplm_dwconv_fwd / nplm_dwconv_bwd, with geometry overrides. An override the
 // build does not hold a kernel for yields -NPLM_DWCONV_ETUNING.
@@ -84,7 +85,7 @@ struct ConvPtrs {
 // Which LDS kernel shape to launch (all are template parameters of the kernels).
 struct LdsShapeSel {
     bool bf16;
-    int vec, rw, nrg, ncw, nwl;
+    int vec, rw, nrg, ncw, nwl, nbuf;
 };
 #define NPLM_DECLARE_LDS_K(KK)                                                                            \
     hipError_t launch_fwd_lds_k##KK(const LdsShapeSel& sh, const ConvPtrs& p, const LdsGeo& g, dim3 grid, \
@@ -114,21 +115,21 @@ constexpr int max_vec(bool bwd, bool bf16, int K) {
     return bwd ? 4 : 8;
 }
 constexpr int default_unroll(bool bwd, int K, int vec) {
+    (void)bwd;
     if (K >= 15) return 4;
-    if (bwd) return vec >= 4 ? 4 : 8;
     return vec >= 8 ? 4 : 8;
 }
 // LDS-staged kernels are built for K <= 9.
 constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
 // Default shape: 4 wave-columns of 64 lanes x 8 bytes = 2 KiB of a row per block, 2 row groups,
-// 4 loader waves; 16-row tiles forward, 12-row tiles backward (x and dy tiles, double buffered, must
-// fit 160 KiB of LDS).
+// 4 loader waves, 16-row tiles. Forward: two x tiles of 22 rows (88 KiB of LDS). Backward: two
+// (22-row dy tile, 16-row x tile) pairs, 152 KiB of the 160 KiB a CU has.
 constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16) {
-    return LdsShapeSel{bf16, bf16 ? 4 : 2, bwd ? 6 : 8, 2, 4, 4};
+    return LdsShapeSel{bf16, bf16 ? 4 : 2, bwd ? 4 : 8, 2, 4, 4, 2};
 }
 constexpr int default_maxt(bool bwd, int K, int vec) {
-    (void)K; (void)vec;
-    return bwd ? 512 : 256;
+    (void)bwd; (void)K; (void)vec;
+    return 256;
 }
 
 }  // namespace nplm

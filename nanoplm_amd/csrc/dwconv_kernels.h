@@ -222,9 +222,14 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
 // =============================================================================================
 // Backward (fused): dx, plus per-block partial sums of dw and db
 // =============================================================================================
-// Row t contributes   dx[t]   = sum_m w[K-1-m] * dy[t-P+m]   (m over the window, masked)
-//                     dw[k]  += dy[t] * x[t-P+k]             (masked the same way)
-//                     db     += dy[t]
+// Both gradients of row t are written against the SAME window of dy rows t-P .. t+P (slot m holds
+// dy[t-P+m]); only the centre row of x is needed, so x is read without any halo:
+//     dx[t]      = sum_m w[K-1-m] * dy[t-P+m]
+//     dw[K-1-m] += x[t] * dy[t-P+m]          (dw[k] = sum_t x[t] * dy[t-k+P], the same sum as
+//                                             sum_t' dy[t'] * x[t'+k-P] with t = t'+k-P)
+//     db        += dy[t]
+// A tap is masked when row t-P+m lies outside the sequence of row t; the two rows of a product are
+// always in the same sequence or the product is dropped, so the mask is the same in either form.
 // Each wave keeps dw/db for its VEC channels in registers across all its tiles. At the end the bt
 // waves of a block that share a wave-column are summed through LDS in fixed order (token slot
 // 0,1,2,...), and the block writes one slab partial[tb][k][c]. No atomics.
@@ -277,25 +282,22 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
             const int t0 = tile * R;
             const int t1 = (t0 + R < T) ? t0 + R : T;
             const int rb = (t0 - P > 0) ? t0 - P : 0;
-            const rsrc_t rx = rows_rsrc(x, rb, T, row_bytes);
-            const rsrc_t rg = rows_rsrc(dy, rb, T, row_bytes);
+            const rsrc_t rg = rows_rsrc(dy, rb, T, row_bytes);   // dy rows from rb (window with halo)
+            const rsrc_t rx = rows_rsrc(x, t0, T, row_bytes);    // x rows from t0 (centre rows only)
             const rsrc_t ro = rows_rsrc(dx, t0, T, row_bytes);
 
-            float xw[WDW ? RG::RING : 1][VEC];   // x  rows tc-P .. tc+U-1+P
-            float gw[RG::RING][VEC];             // dy rows, same range
+            float gw[RG::RING][VEC];   // slot(ph, j) holds dy row tc - P + j
 #pragma unroll
             for (int j = 0; j < K - 1; ++j) {
-                const int so = (clamp_row(t0 - P + j, T) - rb) * rowb;
                 Row r;
-                if constexpr (WDW) { r.bload(rx, lane_off, so); r.to_f32(xw[RG::slot(0, j)]); }
-                r.bload(rg, lane_off, so); r.to_f32(gw[RG::slot(0, j)]);
+                r.bload(rg, lane_off, (clamp_row(t0 - P + j, T) - rb) * rowb);
+                r.to_f32(gw[RG::slot(0, j)]);
             }
             Row nx[WDW ? U : 1], ng[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int so = (clamp_row(t0 + P + u, T) - rb) * rowb;
-                if constexpr (WDW) nx[u].bload(rx, lane_off, so);
-                ng[u].bload(rg, lane_off, so);
+                ng[u].bload(rg, lane_off, (clamp_row(t0 + P + u, T) - rb) * rowb);
+                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(t0 + u, T) - t0) * rowb);
             }
             sc.locate(cu, S, T, t0, sc.seq);
 
@@ -303,17 +305,17 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
 #pragma unroll
                 for (int ph = 0; ph < RG::NPH; ++ph) {
                     if (tc < t1) {
+                        float xc[WDW ? U : 1][VEC];   // x rows tc .. tc+U-1
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
-                            if constexpr (WDW) nx[u].to_f32(xw[RG::slot(ph, K - 1 + u)]);
                             ng[u].to_f32(gw[RG::slot(ph, K - 1 + u)]);
+                            if constexpr (WDW) nx[u].to_f32(xc[u]);
                         }
                         if (tc + U < t1) {
 #pragma unroll
                             for (int u = 0; u < U; ++u) {
-                                const int so = (clamp_row(tc + U + P + u, T) - rb) * rowb;
-                                if constexpr (WDW) nx[u].bload(rx, lane_off, so);
-                                ng[u].bload(rg, lane_off, so);
+                                ng[u].bload(rg, lane_off, (clamp_row(tc + U + P + u, T) - rb) * rowb);
+                                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(tc + U + u, T) - t0) * rowb);
                             }
                         }
                         sc.advance(cu, S, T, tc);
@@ -321,27 +323,21 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                         if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
 #pragma unroll
                             for (int u = 0; u < U; ++u) {
-                                if constexpr (WDW) {
-                                    float gc[VEC];
+                                float acc[VEC];
 #pragma unroll
-                                    for (int v = 0; v < VEC; ++v) { gc[v] = gw[RG::slot(ph, u + P)][v]; dba[v] += gc[v]; }
-#pragma unroll
-                                    for (int k = 0; k < K; ++k)
-#pragma unroll
-                                        for (int v = 0; v < VEC; ++v)
-                                            dwa[v][k] = __builtin_fmaf(gc[v], xw[RG::slot(ph, u + k)][v], dwa[v][k]);
+                                for (int v = 0; v < VEC; ++v) {
+                                    acc[v] = 0.f;
+                                    if constexpr (WDW) dba[v] += gw[RG::slot(ph, u + P)][v];
                                 }
-                                if constexpr (WDX) {
-                                    float acc[VEC];
 #pragma unroll
-                                    for (int v = 0; v < VEC; ++v) acc[v] = 0.f;
+                                for (int m = 0; m < K; ++m)
 #pragma unroll
-                                    for (int m = 0; m < K; ++m)
-#pragma unroll
-                                        for (int v = 0; v < VEC; ++v)
-                                            acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gw[RG::slot(ph, u + m)][v], acc[v]);
-                                    o[u].from_f32(acc);
-                                }
+                                    for (int v = 0; v < VEC; ++v) {
+                                        const float gv = gw[RG::slot(ph, u + m)][v];
+                                        if constexpr (WDX) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
+                                        if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - m]);
+                                    }
+                                if constexpr (WDX) o[u].from_f32(acc);
                             }
                             if constexpr (WDX) {
                                 if (active) {
@@ -355,12 +351,11 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                 const int t = tc + u;
                                 if (t < t1) {
                                     sc.advance(cu, S, T, t);
-                                    float gc[VEC], acc[VEC];
+                                    float acc[VEC];
 #pragma unroll
                                     for (int v = 0; v < VEC; ++v) {
-                                        gc[v] = gw[RG::slot(ph, u + P)][v];
-                                        if constexpr (WDW) dba[v] += gc[v];
                                         acc[v] = 0.f;
+                                        if constexpr (WDW) dba[v] += gw[RG::slot(ph, u + P)][v];
                                     }
 #pragma unroll
                                     for (int m = 0; m < K; ++m) {
@@ -368,14 +363,9 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                         const bool ok = (j >= sc.cs) && (j < sc.ce);
 #pragma unroll
                                         for (int v = 0; v < VEC; ++v) {
-                                            if constexpr (WDW) {
-                                                const float xv = ok ? xw[RG::slot(ph, u + m)][v] : 0.f;
-                                                dwa[v][m] = __builtin_fmaf(gc[v], xv, dwa[v][m]);
-                                            }
-                                            if constexpr (WDX) {
-                                                const float gv = ok ? gw[RG::slot(ph, u + m)][v] : 0.f;
-                                                acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
-                                            }
+                                            const float gv = ok ? gw[RG::slot(ph, u + m)][v] : 0.f;
+                                            if constexpr (WDX) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
+                                            if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - m]);
                                         }
                                     }
                                     if constexpr (WDX) {
@@ -389,10 +379,7 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
 #pragma unroll
                             for (int j = 0; j < K - 1; ++j)
 #pragma unroll
-                                for (int v = 0; v < VEC; ++v) {
-                                    if constexpr (WDW) xw[j][v] = xw[j + U][v];
-                                    gw[j][v] = gw[j + U][v];
-                                }
+                                for (int v = 0; v < VEC; ++v) gw[j][v] = gw[j + U][v];
                         }
                         tc += U;
                     }
@@ -433,14 +420,14 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
 
 // =============================================================================================
 // Finalize: dw[c][k] = sum_p partial[p][k][c], db[c] = sum_p partial[p][K][c], p in fixed order.
-// Block = 64 outputs (adjacent c) x FIN_SPLIT groups of p; each group sums its contiguous share
-// of p in order, then group 0 adds the group sums in order.
+// Block = 64 outputs (adjacent c) x SPLIT groups of p; each group sums its contiguous share of p in
+// order (loads issued 8 at a time), then group 0 adds the group sums in order.
 // =============================================================================================
-constexpr int FIN_SPLIT = 8;
+constexpr int FIN_SPLIT = 16;
 
 template <int SPLIT>
 __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
-                                       float* __restrict__ dw, float* __restrict__ db) {
+                                                                     float* __restrict__ dw, float* __restrict__ db) {
     __shared__ float red[SPLIT][64];
     const int lane = (int)(threadIdx.x & 63);
     const int grp = (int)(threadIdx.x >> 6);
@@ -454,7 +441,15 @@ __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float
     if (on) {
         const float* src = partial + o;
         const size_t stride = (size_t)n_out;
-        for (int p = p0; p < p1; ++p) s += src[(size_t)p * stride];
+        int p = p0;
+        for (; p + 8 <= p1; p += 8) {
+            float t[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) t[i] = src[(size_t)(p + i) * stride];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += t[i];
+        }
+        for (; p < p1; ++p) s += src[(size_t)p * stride];
     }
     red[grp][lane] = s;
     __syncthreads();

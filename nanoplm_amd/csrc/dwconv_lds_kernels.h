@@ -37,7 +37,28 @@ struct LdsGeo {
     int32_t w_bf16;
     int32_t ntiles;     // ceil(T / R)
     int32_t ncb, nbt;   // grid = ncb column blocks x nbt token blocks (nbt <= ntiles)
+    int32_t xcd_group;  // > 0: runs of this many adjacent token-blocks share an XCD (and its L2)
 };
+
+// blockIdx -> (column block, token block). Hardware deals consecutive workgroups round-robin to the
+// 8 XCDs, each with its own L2. With xcd_group = G, the G token-blocks b/8*... of one XCD are
+// adjacent tiles of the same column block, so G-1 of every G halo re-reads hit that XCD's L2 instead
+// of going out to the fabric, while the XCDs still interleave finely (every G tiles) inside the one
+// window of rows the grid is sweeping. Needs nbt % G == 0 and (ncb*nbt/8) % G == 0 (host-checked).
+__device__ __forceinline__ void lds_block_coords(const LdsGeo& g, int& cb, int& tb) {
+    const int b = (int)blockIdx.x;
+    if (g.xcd_group > 0) {
+        const int G = g.xcd_group;
+        const int xcd = b & 7, l = b >> 3;
+        const int k = l / G, r = l - k * G;
+        const int chunk = k * 8 + xcd;
+        cb = chunk % g.ncb;
+        tb = (chunk / g.ncb) * G + r;
+    } else {
+        cb = b % g.ncb;
+        tb = b / g.ncb;
+    }
+}
 
 typedef __attribute__((address_space(3))) void lds_void;
 
@@ -62,23 +83,55 @@ struct LdsShape {
     static_assert(NROWS * CB_BYTES <= 65536, "ds_read immediate offsets are 16 bit");
 };
 
-// Loader: stage rows t0-P .. t0-P+NROWS-1 (clamped to [0,T)) x this block's column block of `src`
-// into `dst` (row pitch CB_BYTES). (row, piece) pairs are dealt round-robin to the loader waves.
+// Loader: stage rows first_row .. first_row+nrows-1 (clamped to [0,T)) x this block's column block of
+// `src` into `dst` (row pitch CB_BYTES). (row, piece) pairs are dealt round-robin to the loader waves.
 template <typename SH>
-__device__ __forceinline__ void stage_tile(const void* __restrict__ src, char* dst, int t0, int T, size_t row_bytes,
-                                           int col_byte0, int valid_bytes, int lw, int nlw, int lane) {
-    const int rb = (t0 - SH::P > 0) ? t0 - SH::P : 0;
+__device__ __forceinline__ void stage_rows(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
+                                           size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw, int lane) {
+    const int rb = first_row > 0 ? first_row : 0;
     const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
     const int rowb = (int)row_bytes;
     const int voff = lane * 16;
-    for (int pair = lw; pair < SH::NROWS * SH::NPIECE; pair += nlw) {
+    for (int pair = lw; pair < nrows * SH::NPIECE; pair += nlw) {
         const int j = pair / SH::NPIECE;
         const int p = pair % SH::NPIECE;
-        const int so = (clamp_row(t0 - SH::P + j, T) - rb) * rowb + col_byte0 + p * 1024;
+        const int so = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0 + p * 1024;
         char* d = dst + j * SH::CB_BYTES + p * 1024;
         if (p * 1024 + voff < valid_bytes)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, voff, so, 0, 0);
     }
+}
+
+// Same as stage_rows, but every loader wave issues exactly CNT loads (surplus slots repeat the last
+// pair, lanes past the end of a narrow column block re-read its last 16 bytes), so that
+// "all but the newest CNT loads have landed" is a compile-time s_waitcnt.
+template <typename SH, int CNT>
+__device__ __forceinline__ void stage_rows_fixed(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
+                                                 size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw,
+                                                 int lane) {
+    const int rb = first_row > 0 ? first_row : 0;
+    const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
+    const int rowb = (int)row_bytes;
+    const int total = nrows * SH::NPIECE;
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+        int pair = lw + i * nlw;
+        pair = pair < total ? pair : total - 1;
+        const int j = pair / SH::NPIECE;
+        const int p = pair % SH::NPIECE;
+        int boff = p * 1024 + lane * 16;
+        boff = boff < valid_bytes ? boff : valid_bytes - 16;
+        const int so = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0;
+        char* d = dst + j * SH::CB_BYTES + p * 1024;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, boff, so, 0, 0);
+    }
+}
+
+// s_waitcnt vmcnt(N) for a compile-time N < 64 (gfx9 encoding: bits 3:0 and 15:14).
+template <int N>
+__device__ __forceinline__ void wait_vmem_but() {
+    static_assert(N >= 0 && N < 64, "vmcnt is 6 bits");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
 template <bool BF16, int VEC>
@@ -116,20 +169,24 @@ __device__ __forceinline__ void wave_bounds(SeqCursor& sc, const int32_t* __rest
 // =============================================================================================
 // Forward
 // =============================================================================================
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL>
+// NBUF = 2: one tile in flight while one is consumed. NBUF = 3: two tiles in flight (the loaders wait
+// only for the older one), which keeps HBM busy when a single tile's latency exceeds its compute time.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, int NBUF>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
                       const void* __restrict__ b, void* __restrict__ y, const LdsGeo g) {
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     using Row = RowVec<BF16, VEC>;
-    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x TILE_BYTES
+    constexpr int CNT = (SH::NROWS * SH::NPIECE + NWL - 1) / NWL;     // loads per loader wave per tile
+    static_assert(NBUF == 2 || NBUF == 3, "two or three tile buffers");
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x TILE_BYTES
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
     const bool is_loader = wv >= SH::NWC;
-    const int cb = (int)blockIdx.x % g.ncb;
-    const int tb = (int)blockIdx.x / g.ncb;
+    int cb, tb;
+    lds_block_coords(g, cb, tb);
     const int T = g.T, S = g.S, C = g.C;
     const size_t row_bytes = (size_t)C * E;
     const int rowb = (int)row_bytes;
@@ -152,8 +209,15 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
     if (is_loader) {
-        stage_tile<SH>(x, lds_raw, tb * R, T, row_bytes, col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
-        wait_vmem_all();
+        stage_rows_fixed<SH, CNT>(x, lds_raw, tb * R - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
+                                  NWL, lane);
+        if (NBUF == 3 && ntl > 1) {
+            stage_rows_fixed<SH, CNT>(x, lds_raw + SH::TILE_BYTES, (tb + g.nbt) * R - P, SH::NROWS, T, row_bytes,
+                                      col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
+            wait_vmem_but<CNT>();     // tile 0 has landed, tile 1 may still be in flight
+        } else {
+            wait_vmem_all();
+        }
     } else {
         load_weights<VEC, K>(w, g.w_bf16, c0, wr);
         if (b) {
@@ -167,13 +231,20 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     __syncthreads();
 
+    int bcur = 0;                       // buffer of tile `it`
     for (int it = 0; it < ntl; ++it) {
         const int t0 = (tb + it * g.nbt) * R;
-        char* cur = lds_raw + (it & 1) * SH::TILE_BYTES;
+        char* cur = lds_raw + bcur * SH::TILE_BYTES;
         if (is_loader) {
-            if (it + 1 < ntl) {
-                stage_tile<SH>(x, lds_raw + ((it + 1) & 1) * SH::TILE_BYTES, t0 + g.nbt * R, T, row_bytes, col_byte0,
-                               valid_bytes, wv - SH::NWC, NWL, lane);
+            // stage tile it + NBUF - 1 into the buffer freed by the barrier that ended iteration it - 1,
+            // then wait until tile it + 1 has landed
+            const int ahead = NBUF - 1;
+            if (it + ahead < ntl) {
+                const int bnew = (bcur + ahead) % NBUF;
+                stage_rows_fixed<SH, CNT>(x, lds_raw + bnew * SH::TILE_BYTES, t0 + ahead * g.nbt * R - P, SH::NROWS, T,
+                                          row_bytes, col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
+                if (NBUF == 3) wait_vmem_but<CNT>(); else wait_vmem_all();
+            } else {
                 wait_vmem_all();
             }
         } else {
@@ -231,29 +302,34 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
             }
         }
         __syncthreads();   // next tile is in LDS; this tile's buffer may be overwritten
+        bcur = (bcur + 1 == NBUF) ? 0 : bcur + 1;
     }
 }
 
 // =============================================================================================
 // Backward (fused)
 // =============================================================================================
-// LDS: [2 buffers][x tile, dy tile]; without dw/db (WDW = false) only the dy tiles are staged.
+// Same arithmetic as the sliding-window backward: both gradients of row t read the one window of dy
+// rows t-P .. t+P, and x only contributes its centre row:
+//     dx[t] = sum_m w[K-1-m] * dy[t-P+m],   dw[K-1-m] += x[t] * dy[t-P+m],   db += dy[t].
+// So only the dy tile carries halo rows; the x tile is exactly the R rows of the tile.
+// LDS: [2 buffers][dy tile (R+K-1 rows), x tile (R rows, only when dw/db are wanted)].
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                       const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
-    constexpr int NTENS = WDW ? 2 : 1;
-    constexpr int BUF_BYTES = NTENS * SH::TILE_BYTES;
+    constexpr int XT_BYTES = R * SH::CB_BYTES;
+    constexpr int BUF_BYTES = SH::TILE_BYTES + (WDW ? XT_BYTES : 0);
     using Row = RowVec<BF16, VEC>;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
     const bool is_loader = wv >= SH::NWC;
-    const int cb = (int)blockIdx.x % g.ncb;
-    const int tb = (int)blockIdx.x / g.ncb;
+    int cb, tb;
+    lds_block_coords(g, cb, tb);
     const int T = g.T, S = g.S, C = g.C;
     const size_t row_bytes = (size_t)C * E;
     const int rowb = (int)row_bytes;
@@ -271,15 +347,14 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     const int out_voff = c0 * E;
     const int lw = wv - SH::NWC;
 
-    // buffer layout: dy tile first, then (if staged) the x tile
     auto stage_both = [&](char* buf, int t0) {
-        // loader waves split the two tensors between them when there are at least two of them
+        // with two or more loader waves, even ones take the dy tile and odd ones the x tile
         if constexpr (WDW && NWL >= 2) {
-            if (lw & 1) stage_tile<SH>(x, buf + SH::TILE_BYTES, t0, T, row_bytes, col_byte0, valid_bytes, lw >> 1, NWL / 2, lane);
-            else        stage_tile<SH>(dy, buf, t0, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane);
+            if (lw & 1) stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, row_bytes, col_byte0, valid_bytes, lw >> 1, NWL / 2, lane);
+            else        stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane);
         } else {
-            stage_tile<SH>(dy, buf, t0, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
-            if constexpr (WDW) stage_tile<SH>(x, buf + SH::TILE_BYTES, t0, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+            stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+            if constexpr (WDW) stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
         }
     };
 
@@ -316,20 +391,17 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 WaveBounds<RW> wb;
                 wave_bounds<RW, P>(sc, cu, S, T, tf, wb);
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
-                const char* lpg = cur + loff;
-                const char* lpx = cur + SH::TILE_BYTES + loff;
-                // centre dy rows of the wave's outputs (staged row u + P); rows past T contribute nothing
-                float gc[WDW ? RW : 1][VEC];
+                const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
+                const char* lpx = cur + SH::TILE_BYTES + loff;     // x : staged row u <-> global row tf + u
+                float xc[WDW ? RW : 1][VEC];
                 if constexpr (WDW) {
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
-                        lds_read_row<BF16, VEC>(lpg + (u + P) * SH::CB_BYTES, gc[u]);
-                        if (tf + u >= T) {
+                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
+                        if (tf + u >= T) {     // rows past the end contribute nothing
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) gc[u][v] = 0.f;
+                            for (int v = 0; v < VEC; ++v) xc[u][v] = 0.f;
                         }
-#pragma unroll
-                        for (int v = 0; v < VEC; ++v) dba[v] += gc[u][v];
                     }
                 }
                 float acc[WDX ? RW : 1][VEC];
@@ -342,16 +414,21 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 if (wb.interior) {
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
-                        float xr[VEC], gr[VEC];
-                        if constexpr (WDW) lds_read_row<BF16, VEC>(lpx + j * SH::CB_BYTES, xr);
-                        if constexpr (WDX) lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        float gr[VEC];
+                        lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        if constexpr (WDW) {
+                            if (j >= P && j < P + RW) {   // centre row of output j - P (interior: always < T)
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) dba[v] += gr[v];
+                            }
+                        }
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) {
-                                    if constexpr (WDW) dwa[v][j - u] = __builtin_fmaf(gc[u][v], xr[v], dwa[v][j - u]);
                                     if constexpr (WDX) acc[u][v] = __builtin_fmaf(wr[v][K - 1 - (j - u)], gr[v], acc[u][v]);
+                                    if constexpr (WDW) dwa[v][K - 1 - (j - u)] = __builtin_fmaf(xc[u][v], gr[v], dwa[v][K - 1 - (j - u)]);
                                 }
                             }
                         }
@@ -359,24 +436,24 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 } else {
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
-                        float xr[VEC], gr[VEC];
-                        if constexpr (WDW) lds_read_row<BF16, VEC>(lpx + j * SH::CB_BYTES, xr);
-                        if constexpr (WDX) lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        float gr[VEC];
+                        lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
                         const int grow = tf - P + j;
+                        if constexpr (WDW) {
+                            if (j >= P && j < P + RW && grow < T) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) dba[v] += gr[v];
+                            }
+                        }
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
                                 const bool ok = (grow >= wb.lo[u]) && (grow < wb.hi[u]);
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) {
-                                    if constexpr (WDW) {
-                                        const float xv = ok ? xr[v] : 0.f;
-                                        dwa[v][j - u] = __builtin_fmaf(gc[u][v], xv, dwa[v][j - u]);
-                                    }
-                                    if constexpr (WDX) {
-                                        const float gv = ok ? gr[v] : 0.f;
-                                        acc[u][v] = __builtin_fmaf(wr[v][K - 1 - (j - u)], gv, acc[u][v]);
-                                    }
+                                    const float gv = ok ? gr[v] : 0.f;
+                                    if constexpr (WDX) acc[u][v] = __builtin_fmaf(wr[v][K - 1 - (j - u)], gv, acc[u][v]);
+                                    if constexpr (WDW) dwa[v][K - 1 - (j - u)] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - (j - u)]);
                                 }
                             }
                         }
