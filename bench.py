@@ -149,8 +149,6 @@ def main():
     ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     cu, w, b = d.cu_seqlens, d.weight, d.bias
-    tune = _lib.Tuning()
-
     def fwd(i):
         j = i % NSET
         _lib.check(lib.nplm_dwconv_fwd(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(), ys[j].data_ptr(),
@@ -181,22 +179,28 @@ def main():
     tokens_per_s = T / (ms_per_step / 1e3)
 
     # ---- per-kernel durations with HIP events on the launch stream ---------------------------------
+    # One set of four events per step, recorded back to back like the timed loop above (no host
+    # synchronisation between steps), read after a single synchronise at the end.
     n_ev = min(max(args.steps, 10), 100)
-    ev = HipEvents(4)
-    tune.mid_event = ev.ev[2]
-    fwd_us, bwd_us, fin_us = [], [], []
+    evs = [HipEvents(4) for _ in range(n_ev)]
+    tunes = []
     for i in range(n_ev):
-        ev.record(0, stream)
+        t = _lib.Tuning()
+        t.mid_event = evs[i].ev[2]
+        tunes.append(t)
+    for i in range(n_ev):
+        e = evs[i]
+        e.record(0, stream)
         fwd(i)
-        ev.record(1, stream)
+        e.record(1, stream)
         if fwd_bwd:
-            bwd(i, tune)            # records event 2 between the fused kernel and the finalize kernel
-            ev.record(3, stream)
-        torch.cuda.synchronize()
-        fwd_us.append(ev.elapsed_us(0, 1))
-        if fwd_bwd:
-            bwd_us.append(ev.elapsed_us(1, 2))
-            fin_us.append(ev.elapsed_us(2, 3))
+            bwd(i, tunes[i])        # records event 2 between the fused kernel and the finalize kernel
+            e.record(3, stream)
+    torch.cuda.synchronize()
+    fwd_us = [e.elapsed_us(0, 1) for e in evs]
+    bwd_us = [e.elapsed_us(1, 2) for e in evs] if fwd_bwd else []
+    fin_us = [e.elapsed_us(2, 3) for e in evs] if fwd_bwd else []
+    ev = evs[0]
     fwd_avg = statistics.fmean(fwd_us)
     fwd_bytes = wl.algorithmic_bytes("fwd")
 

@@ -116,7 +116,7 @@ constexpr int max_vec(bool bwd, bool bf16, int K) {
 }
 constexpr int default_unroll(bool bwd, int K, int vec) {
     (void)bwd;
-    if (K >= 15) return 4;
+    if (K >= 15) return 8;
     return vec >= 8 ? 4 : 8;
 }
 // LDS-staged kernels are built for K <= 9.

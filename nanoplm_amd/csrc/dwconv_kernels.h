@@ -23,6 +23,8 @@
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); the tensor
 // contract is the packed path's: modeling.py:339,421-439 and collator.py:322-325,405-458.
 #pragma once
+#include <utility>
+
 #include "dwconv_device.h"
 
 namespace nplm {
@@ -71,6 +73,17 @@ __device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_b
 #pragma unroll
             for (int k = 0; k < K; ++k) wr[v][k] = wp[v * K + k];
     }
+}
+
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N-1>{}).
+// Used where a loop variable must be a constant expression (register-ring slot numbers).
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, static_cast<F&&>(f));
 }
 
 __device__ __forceinline__ int clamp_row(int r, int T) { return r < 0 ? 0 : (r >= T ? T - 1 : r); }
@@ -151,9 +164,10 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
         for (int u = 0; u < U; ++u) nxt[u].bload(rx, lane_off, (clamp_row(t0 + P + u, T) - rb) * rowb);
         sc.locate(cu, S, T, t0, sc.seq);
 
-        for (int tc = t0; tc < t1;) {
-#pragma unroll
-            for (int ph = 0; ph < RG::NPH; ++ph) {
+        int tc = t0;
+        while (tc < t1) {
+            static_for<RG::NPH>([&](auto ph_c) {
+                constexpr int ph = decltype(ph_c)::value;
                 if (tc < t1) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) nxt[u].to_f32(win[RG::slot(ph, K - 1 + u)]);
@@ -214,7 +228,7 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
                     }
                     tc += U;
                 }
-            }
+            });
         }
     }
 }
@@ -301,9 +315,10 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
             }
             sc.locate(cu, S, T, t0, sc.seq);
 
-            for (int tc = t0; tc < t1;) {
-#pragma unroll
-                for (int ph = 0; ph < RG::NPH; ++ph) {
+            int tc = t0;
+            while (tc < t1) {
+                static_for<RG::NPH>([&](auto ph_c) {
+                    constexpr int ph = decltype(ph_c)::value;
                     if (tc < t1) {
                         float xc[WDW ? U : 1][VEC];   // x rows tc .. tc+U-1
 #pragma unroll
@@ -383,7 +398,7 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                         }
                         tc += U;
                     }
-                }
+                });
             }
         }
     }
