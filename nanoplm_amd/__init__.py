@@ -6,7 +6,10 @@ from .dwconv import (  # noqa: F401
     check_cu_seqlens,
     varlen_dwconv,
     varlen_dwconv_bwd,
+    varlen_dwconv_bwd_op,
+    varlen_dwconv_compilable,
     varlen_dwconv_fwd,
+    varlen_dwconv_fwd_op,
 )
 
 __version__ = "0.1.0"

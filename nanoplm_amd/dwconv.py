@@ -185,7 +185,64 @@ class VarlenDWConv1d(nn.Module):
             nn.init.normal_(self.bias, mean=0.0, std=0.02)
 
     def forward(self, x: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
+        if torch.compiler.is_compiling():
+            # under torch.compile the opaque custom ops keep the graph whole
+            return varlen_dwconv_fwd_op(x, cu_seqlens, self.weight, self.bias)
         return VarlenDWConv1dFunction.apply(x, cu_seqlens, self.weight, self.bias)
 
     def extra_repr(self) -> str:
         return f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}"
+
+
+# ---------------------------------------------------------------------------------------------
+# torch.library registration: the same two kernels as opaque custom ops, so that
+# torch.compile(model, dynamic=False) (src/nanoplm/pretraining/pure_pipeline.py:519-524) traces
+# through a model that contains the conv without a graph break. Neither op synchronises the host;
+# cu_seqlens may be the static collator's fixed-length tensor (collator.py:430-450).
+# ---------------------------------------------------------------------------------------------
+@torch.library.custom_op("nanoplm_amd::varlen_dwconv_fwd", mutates_args=(), device_types="cuda")
+def varlen_dwconv_fwd_op(x: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
+                         bias: Optional[torch.Tensor]) -> torch.Tensor:
+    return varlen_dwconv_fwd(x, cu_seqlens, weight, bias)
+
+
+@varlen_dwconv_fwd_op.register_fake
+def _(x, cu_seqlens, weight, bias):
+    return torch.empty_like(x, memory_format=torch.contiguous_format)
+
+
+@torch.library.custom_op("nanoplm_amd::varlen_dwconv_bwd", mutates_args=(), device_types="cuda")
+def varlen_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor,
+                         weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dw, db) with dw [C,K] and db [C] in fp32."""
+    dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight)
+    return dx, dw, db
+
+
+@varlen_dwconv_bwd_op.register_fake
+def _(x, dy, cu_seqlens, weight):
+    C, K = weight.shape
+    return (torch.empty_like(x, memory_format=torch.contiguous_format),
+            x.new_empty((C, K), dtype=torch.float32), x.new_empty((C,), dtype=torch.float32))
+
+
+def _op_setup_context(ctx, inputs, output):
+    x, cu_seqlens, weight, bias = inputs
+    ctx.save_for_backward(x, cu_seqlens, weight)
+    ctx.bias_dtype = None if bias is None else bias.dtype
+
+
+def _op_backward(ctx, dy):
+    x, cu_seqlens, weight = ctx.saved_tensors
+    if dy.dtype != x.dtype:
+        dy = dy.to(x.dtype)
+    dx, dw, db = varlen_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, weight)
+    return dx, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype))
+
+
+varlen_dwconv_fwd_op.register_autograd(_op_backward, setup_context=_op_setup_context)
+
+
+def varlen_dwconv_compilable(x, cu_seqlens, weight, bias=None):
+    """Same result as :func:`varlen_dwconv`, routed through the registered custom ops (traceable)."""
+    return varlen_dwconv_fwd_op(x, cu_seqlens, weight, bias)

@@ -87,3 +87,45 @@ def test_runs_on_a_side_stream():
     dx0, dw0, db0 = npa.varlen_dwconv_bwd(wl.x, wl.dy, wl.cu_seqlens, wl.weight)
     torch.cuda.synchronize()
     assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1) and torch.equal(db0, db1)
+
+
+def test_registered_custom_ops_pass_opcheck_and_compile_without_graph_breaks():
+    """torch.compile(dynamic=False) is how the reference runs its model
+    (src/nanoplm/pretraining/pure_pipeline.py:519-524); the conv must trace as one opaque op and accept
+    the static collator's fixed-length cu_seqlens (collator.py:430-450)."""
+    from nanoplm_amd.workloads import static_packed_cu
+
+    wl = make_workload(2, T=3000, C=256, with_dy=True)
+    F, W = 4096, 512
+    cu = static_packed_cu(wl.cu_seqlens, F, W, cu_len=64).to(DEV)
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(F, 256, generator=g).bfloat16().to(DEV)
+    dy = torch.randn(F, 256, generator=g).bfloat16().to(DEV)
+    torch.library.opcheck(npa.varlen_dwconv_fwd_op, (x, cu, wl.weight.to(DEV), wl.bias.to(DEV)),
+                          test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(npa.varlen_dwconv_bwd_op, (x, dy, cu, wl.weight.to(DEV)),
+                          test_utils=("test_schema", "test_faketensor"))
+
+    conv = npa.VarlenDWConv1d(256, 7).to(DEV).to(torch.bfloat16)
+    with torch.no_grad():
+        conv.weight.copy_(wl.weight.to(DEV))
+        conv.bias.copy_(wl.bias.to(DEV))
+
+    def run(mod):
+        xin = x.clone().requires_grad_(True)
+        for p in conv.parameters():
+            p.grad = None
+        y = mod(xin, cu)
+        (y.float() * dy.float()).sum().backward()
+        return y.detach(), xin.grad, conv.weight.grad.clone(), conv.bias.grad.clone()
+
+    y0, dx0, dw0, db0 = run(conv)
+    compiled = torch.compile(conv, backend="aot_eager", fullgraph=True, dynamic=False)
+    y1, dx1, dw1, db1 = run(compiled)
+    assert torch.equal(y0, y1) and torch.equal(dx0, dx1) and torch.equal(dw0, dw1) and torch.equal(db0, db1)
+    # and against the oracle on the real (unpadded) part
+    T = wl.T
+    cu_host = cu.cpu()
+    y64 = O.c_oracle_fwd(x.cpu(), cu_host, wl.weight, wl.bias)
+    assert_act_close(y1, y64, torch.bfloat16, "compiled y")
+    assert T < F

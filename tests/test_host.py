@@ -215,3 +215,37 @@ def test_algorithmic_bytes_of_the_headline_config():
     assert w3.algorithmic_bytes("bwd") == 3 * T * C * e + C * K * e + 4 * C * (K + 1) + 4 * (S + 1)
     # at C=1024: 5*T*C*e = 1 342 177 280
     assert 5 * 131072 * 1024 * 2 == 1342177280
+
+
+# ---- torch.library registration (traceability; no kernel is run) ------------------------------------
+def test_custom_ops_trace_with_fake_tensors():
+    """Schemas and fake (shape/dtype) implementations of the registered ops, without a GPU. The autograd
+    formula needs a device context and is exercised by the GPU tests."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.fx.experimental.proxy_tensor import make_fx
+
+    assert str(torch.ops.nanoplm_amd.varlen_dwconv_fwd.default._schema) == (
+        "nanoplm_amd::varlen_dwconv_fwd(Tensor x, Tensor cu_seqlens, Tensor weight, Tensor? bias) -> Tensor")
+    assert str(torch.ops.nanoplm_amd.varlen_dwconv_bwd.default._schema) == (
+        "nanoplm_amd::varlen_dwconv_bwd(Tensor x, Tensor dy, Tensor cu_seqlens, Tensor weight) -> (Tensor, Tensor, Tensor)")
+    with FakeTensorMode():
+        x = torch.empty(100, 64, dtype=torch.bfloat16, device="cuda")
+        cu = torch.empty(5, dtype=torch.int32, device="cuda")
+        w = torch.empty(64, 7, dtype=torch.float32, device="cuda")
+        b = torch.empty(64, dtype=torch.float32, device="cuda")
+        y = nanoplm_amd.varlen_dwconv_compilable(x, cu, w, b)
+        assert y.shape == x.shape and y.dtype == torch.bfloat16 and y.device.type == "cuda"
+        dx, dw, db = nanoplm_amd.varlen_dwconv_bwd_op(x, y, cu, w)
+        assert dx.shape == x.shape and dx.dtype == torch.bfloat16
+        assert dw.shape == (64, 7) and dw.dtype == torch.float32 and db.shape == (64,) and db.dtype == torch.float32
+
+    def f(x, cu, w):
+        y = nanoplm_amd.varlen_dwconv_compilable(x, cu, w, None)
+        return nanoplm_amd.varlen_dwconv_bwd_op(x, y, cu, w)
+
+    with FakeTensorMode(allow_non_fake_inputs=True):
+        args = (torch.empty(32, 16, device="cuda"), torch.empty(3, dtype=torch.int32, device="cuda"),
+                torch.empty(16, 3, device="cuda"))
+        gm = make_fx(f, tracing_mode="fake")(*args)
+    targets = {str(n.target) for n in gm.graph.nodes if n.op == "call_function"}
+    assert "nanoplm_amd.varlen_dwconv_fwd.default" in targets and "nanoplm_amd.varlen_dwconv_bwd.default" in targets
