@@ -233,14 +233,15 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
 }
 
 // algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged.
-// Measured on MI355X at T=131072, C=1024, K=7, bf16: the forward is fastest LDS-staged; the backward
-// keeps two tensors with halos in flight, which LDS (160 KiB per CU) cannot hold twice over, so the
-// register-resident sliding-window kernel wins there.
+// Measured on MI355X at T=131072, C=1024, K=7, bf16: both passes are fastest LDS-staged (the chip
+// sweeps one compact window of rows with every load of a tile issued at once); the sliding-window
+// kernels take what the LDS kernels are not built for (K > 9, narrow or unaligned rows).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    (void)bwd;
     const bool ok = lds_eligible(bf16, T, C, K, align_bits);
     if (tune && tune->algo == 2) return ok ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
-    return (ok && !bwd) ? 2 : 1;
+    return ok ? 2 : 1;
 }
 
 // 256 threads x 4 x 16 B = one contiguous 16 KiB chunk per block
@@ -469,9 +470,16 @@ int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const
 size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    // enough for whichever kernel family the library picks for these sizes (the choice also depends
+    // on pointer alignment, which is not known here)
     Plan p;
     if (make_plan(true, bf16, T, C, K, 0, nullptr, &p)) return 0;
-    const size_t bytes = (size_t)p.nbt * (K + 1) * C * sizeof(float);
+    int slabs = p.nbt;
+    if (lds_eligible(bf16, T, C, K, 0)) {
+        LdsPlan lp;
+        if (make_lds_plan(true, bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
+    }
+    const size_t bytes = (size_t)slabs * (K + 1) * C * sizeof(float);
     return (bytes + 255) & ~(size_t)255;
 }
 

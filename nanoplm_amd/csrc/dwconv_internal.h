@@ -121,11 +121,15 @@ constexpr int default_unroll(bool bwd, int K, int vec) {
 }
 // LDS-staged kernels are built for K <= 9.
 constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
-// Default shape: 4 wave-columns of 64 lanes x 8 bytes = 2 KiB of a row per block, 2 row groups,
-// 4 loader waves, 16-row tiles. Forward: two x tiles of 22 rows (88 KiB of LDS). Backward: two
-// (22-row dy tile, 16-row x tile) pairs, 152 KiB of the 160 KiB a CU has.
+// Default shapes (a block always owns 2 KiB of every row of its tile, 16-row tiles):
+//   forward : 4 wave-columns x 8 bytes per lane, 2 row groups of 8 rows, 4 loader waves; two x tiles
+//             of 16 + K-1 rows (88 KiB of LDS at K = 7).
+//   backward: 8 wave-columns x 4 bytes per lane, 1 row group of 16 rows, 8 loader waves; two
+//             (dy tile of 16 + K-1 rows, x tile of 16 rows) pairs = 152 KiB of the 160 KiB a CU has
+//             (exactly 160 KiB at K = 9). Four bytes per lane keep the 16-row register tile
+//             (dx accumulators + x rows + weights + dw/db) under the 128 registers 16 waves leave.
 constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16) {
-    return LdsShapeSel{bf16, bf16 ? 4 : 2, bwd ? 4 : 8, 2, 4, 4, 2};
+    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, 8, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
 }
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)bwd; (void)K; (void)vec;

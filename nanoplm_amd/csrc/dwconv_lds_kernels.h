@@ -22,6 +22,13 @@
 // across all tiles of the block and are combined as in the sliding-window kernels (row groups summed
 // through LDS in fixed order, one slab per token-block, then dwconv_finalize_kernel). No atomics.
 //
+// Sequence boundaries: the cursor lookup for the NEXT tile (a chain of dependent scalar loads) runs
+// right before the tile barrier, where the compute waves would otherwise idle. A wave whose rows and
+// taps all lie in one sequence takes an unmasked path. A wave that touches a boundary keeps the
+// same unrolled schedule and selects every tap by a bit of its output row's tap mask; that path
+// must stay close to the unmasked one in cost, because tiles are dealt to blocks statically and a
+// block's time is the sum of its tiles: a slow boundary path shows up as a long tail of the grid.
+//
 // Every wave of a block executes exactly the same sequence of barriers: the trip counts depend only
 // on blockIdx and the launch geometry.
 //
@@ -144,25 +151,62 @@ __device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
 // Per-output-row tap limits of a wave's RW rows: tap row g is valid for output u iff lo[u] <= g < hi[u].
 template <int RW>
 struct WaveBounds {
-    bool interior;   // every tap of every row of the wave lies inside one sequence
     int lo[RW], hi[RW];
 };
 
+// The expensive half of the boundary lookup: position the cursor on the sequence of row tf (a chain
+// of dependent scalar loads). The compute waves run it for the NEXT tile right before the tile
+// barrier, where they would otherwise idle until the loaders' data has landed.
+// Returns true when every tap of rows tf .. tf+RW-1 lies inside that one sequence.
 template <int RW, int P>
-__device__ __forceinline__ void wave_bounds(SeqCursor& sc, const int32_t* __restrict__ cu, int S, int T, int tf,
-                                            WaveBounds<RW>& wb) {
-    // tf = first output row of the wave (tf < T)
+__device__ __forceinline__ bool wave_locate(SeqCursor& sc, const int32_t* __restrict__ cu, int S, int T, int tf) {
+    if (tf >= T) return true;
     sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
     const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
-    wb.interior = (tf - P >= sc.cs) && (tl + P < sc.ce);
-    if (!wb.interior) {
+    return (tf - P >= sc.cs) && (tl + P < sc.ce);
+}
+
+// The cheap half, only needed for a wave whose rows touch a sequence boundary: walk the cursor over
+// the RW rows. `sc` is taken by value so the caller's cursor keeps pointing at row tf.
+template <int RW>
+__device__ __forceinline__ void wave_row_bounds(SeqCursor sc, const int32_t* __restrict__ cu, int S, int T, int tf,
+                                                WaveBounds<RW>& wb) {
 #pragma unroll
-        for (int u = 0; u < RW; ++u) {
-            const int t = tf + u;
-            if (t < T) sc.advance(cu, S, T, t);
-            wb.lo[u] = sc.cs;
-            wb.hi[u] = sc.ce;
+    for (int u = 0; u < RW; ++u) {
+        const int t = tf + u;
+        if (t < T) sc.advance(cu, S, T, t);
+        wb.lo[u] = sc.cs;
+        wb.hi[u] = sc.ce;
+    }
+}
+
+// Empty volatile asm that takes N registers in and out: orders the instructions that produce them
+// before everything that follows (and compiler-level memory accesses do not move across it).
+template <int N>
+__device__ __forceinline__ void pin_regs(float (&r)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) asm volatile("" : "+v"(r[i]) : : "memory");
+}
+
+// Tap masks of a wave's RW output rows, for a wave whose rows touch a sequence boundary: bit m of
+// vm[u] is set iff tap row (tf + u) - P + m lies inside the sequence of output row tf + u. Rows past
+// the end of the tensor get an empty mask. `sc` (by value) must be positioned on row tf.
+template <int RW, int K>
+__device__ __forceinline__ void wave_tap_masks(SeqCursor sc, const int32_t* __restrict__ cu, int S, int T, int tf,
+                                               uint32_t (&vm)[RW]) {
+    constexpr int P = (K - 1) / 2;
+#pragma unroll
+    for (int u = 0; u < RW; ++u) {
+        const int t = tf + u;
+        uint32_t m = 0;
+        if (t < T) {
+            sc.advance(cu, S, T, t);
+            int lo = sc.cs - (t - P), hi = sc.ce - (t - P);     // valid taps: lo <= m < hi
+            lo = lo < 0 ? 0 : lo;
+            hi = hi > K ? K : hi;
+            if (hi > lo) m = (uint32_t)(((1ull << hi) - 1ull) & ~((1ull << lo) - 1ull));
         }
+        vm[u] = m;
     }
 }
 
@@ -229,6 +273,8 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     }
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    bool interior = true;               // bounds of the wave's rows in the tile about to be computed
+    if (!is_loader) interior = wave_locate<RW, P>(sc, cu, S, T, tb * R + rg * RW);
     __syncthreads();
 
     int bcur = 0;                       // buffer of tile `it`
@@ -250,15 +296,13 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
         } else {
             const int tf = t0 + rg * RW;
             if (tf < T) {
-                WaveBounds<RW> wb;
-                wave_bounds<RW, P>(sc, cu, S, T, tf, wb);
                 float acc[RW][VEC];
 #pragma unroll
                 for (int u = 0; u < RW; ++u)
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[u][v] = bias[v];
                 const char* lp = cur + (rg * RW) * SH::CB_BYTES + lc0 * E;
-                if (wb.interior) {
+                if (interior) {
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
@@ -272,6 +316,8 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         }
                     }
                 } else {
+                    WaveBounds<RW> wb;
+                    wave_row_bounds<RW>(sc, cu, S, T, tf, wb);
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
@@ -300,6 +346,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         if (tf + u < T) o[u].bstore(ry, out_voff, u * rowb);
                 }
             }
+            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, cu, S, T, t0 + g.nbt * R + rg * RW);
         }
         __syncthreads();   // next tile is in LDS; this tile's buffer may be overwritten
         bcur = (bcur + 1 == NBUF) ? 0 : bcur + 1;
@@ -375,6 +422,8 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     }
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    bool interior = true;
+    if (!is_loader) interior = wave_locate<RW, P>(sc, cu, S, T, tb * R + rg * RW);
     __syncthreads();
 
     for (int it = 0; it < ntl; ++it) {
@@ -388,30 +437,29 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         } else {
             const int tf = t0 + rg * RW;
             if (tf < T) {
-                WaveBounds<RW> wb;
-                wave_bounds<RW, P>(sc, cu, S, T, tf, wb);
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
                 const char* lpx = cur + SH::TILE_BYTES + loff;     // x : staged row u <-> global row tf + u
-                float xc[WDW ? RW : 1][VEC];
-                if constexpr (WDW) {
+                const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
+                if (interior) {
+                    float xc[WDW ? RW : 1][VEC];
+                    if constexpr (WDW) {
 #pragma unroll
-                    for (int u = 0; u < RW; ++u) {
-                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
-                        if (tf + u >= T) {     // rows past the end contribute nothing
+                        for (int u = 0; u < RW; ++u) {
+                            lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
+                            if (tf + u >= T) {     // rows past the end contribute nothing
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) xc[u][v] = 0.f;
+                                for (int v = 0; v < VEC; ++v) xc[u][v] = 0.f;
+                            }
                         }
                     }
-                }
-                float acc[WDX ? RW : 1][VEC];
-                if constexpr (WDX) {
+                    float acc[WDX ? RW : 1][VEC];
+                    if constexpr (WDX) {
 #pragma unroll
-                    for (int u = 0; u < RW; ++u)
+                        for (int u = 0; u < RW; ++u)
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) acc[u][v] = 0.f;
-                }
-                if (wb.interior) {
+                            for (int v = 0; v < VEC; ++v) acc[u][v] = 0.f;
+                    }
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float gr[VEC];
@@ -433,22 +481,53 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             }
                         }
                     }
+                    if constexpr (WDX) {
+                        Row o[RW];
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                        if (active) {
+#pragma unroll
+                            for (int u = 0; u < RW; ++u)
+                                if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
+                        }
+                    }
                 } else {
+                    // A sequence boundary falls inside the wave's window: same unrolled schedule, every
+                    // tap selected (never multiplied by 0) by bit m of its output row's tap mask.
+                    uint32_t vm[RW];
+                    wave_tap_masks<RW, K>(sc, cu, S, T, tf, vm);
+                    float xc[WDW ? RW : 1][VEC];
+                    if constexpr (WDW) {
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
+                    }
+                    float acc[WDX ? RW : 1][VEC];
+                    if constexpr (WDX) {
+#pragma unroll
+                        for (int u = 0; u < RW; ++u)
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) acc[u][v] = 0.f;
+                    }
+                    // one staged row ahead in registers; the scheduling fences keep the (already rare)
+                    // path from hoisting every read and mask to the top and running out of registers
+                    Row nxt;
+                    nxt.load(lpg);
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float gr[VEC];
-                        lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
-                        const int grow = tf - P + j;
+                        nxt.to_f32(gr);
+                        if (j + 1 < RW + K - 1) nxt.load(lpg + (j + 1) * SH::CB_BYTES);
                         if constexpr (WDW) {
-                            if (j >= P && j < P + RW && grow < T) {
+                            if (j >= P && j < P + RW) {   // centre tap of output j - P: valid iff that row exists
+                                const bool okc = (vm[j - P] >> P) & 1u;
 #pragma unroll
-                                for (int v = 0; v < VEC; ++v) dba[v] += gr[v];
+                                for (int v = 0; v < VEC; ++v) dba[v] += okc ? gr[v] : 0.f;
                             }
                         }
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
-                                const bool ok = (grow >= wb.lo[u]) && (grow < wb.hi[u]);
+                                const bool ok = (vm[u] >> (j - u)) & 1u;
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) {
                                     const float gv = ok ? gr[v] : 0.f;
@@ -457,20 +536,31 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                 }
                             }
                         }
+                        // pin this row's arithmetic here: every accumulator passes through an empty
+                        // volatile asm, so nothing of row j can sink below the read of row j + 2
+                        if constexpr (WDX) {
+#pragma unroll
+                            for (int u = 0; u < RW; ++u)
+                                if (j - u >= 0 && j - u < K) pin_regs<VEC>(acc[u]);
+                        }
+                        if constexpr (WDW) {
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) pin_regs<K>(dwa[v]);
+                        }
                     }
-                }
-                if constexpr (WDX) {
-                    const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
-                    Row o[RW];
+                    if constexpr (WDX) {
+                        Row o[RW];
 #pragma unroll
-                    for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
-                    if (active) {
+                        for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                        if (active) {
 #pragma unroll
-                        for (int u = 0; u < RW; ++u)
-                            if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
+                            for (int u = 0; u < RW; ++u)
+                                if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
+                        }
                     }
                 }
             }
+            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, cu, S, T, t0 + g.nbt * R + rg * RW);
         }
         __syncthreads();
     }
