@@ -567,10 +567,22 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 
     if constexpr (!WDW) return;
 
+    float* slab = partial + (size_t)tb * (K + 1) * C;
+    if constexpr (NRG == 1) {
+        // one row group: every (tap, channel) sum of the block already sits in exactly one lane
+        if (active) {
+#pragma unroll
+            for (int kk = 0; kk <= K; ++kk) {
+                float* dst = slab + (size_t)kk * C + c0;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) dst[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : dba[v];
+            }
+        }
+        return;
+    }
     // ---- block-level pass: sum the NRG row groups of each wave-column, group order 0,1,2,... ----
     // (the tiles are dead after the last barrier above; loader waves only keep the barriers company)
     float* red = reinterpret_cast<float*>(lds_raw);   // [NWC][VEC][64]
-    float* slab = partial + (size_t)tb * (K + 1) * C;
 #pragma unroll
     for (int kk = 0; kk <= K; ++kk) {
         float val[VEC];
