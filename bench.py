@@ -14,6 +14,8 @@ One JSON line is printed:
   roofline      the dominant kernel (the fused backward): algorithmic bytes per launch divided by its
                 average duration, measured with HIP events recorded on the launch stream
   roofline_fwd  the same for the forward kernel (informational)
+  back_to_back_us  span of 30 consecutive launches of one pass divided by 30 (informational: an event
+                record ends a kernel with a cache write-back that consecutive launches overlap)
   cpu_baseline  the reference path (per-sequence torch conv1d + autograd, oracle/dwconv_ref.py) timed
                 on this box's host cores on a bounded sample of the same workload
 """
@@ -36,8 +38,8 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
 # scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
 # profiles/): keyed by (workload name, kernel).
 MEASURED_TRAFFIC = {
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 550166591,    # 1.025 x algorithmic
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 835409445,   # 1.037 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 550192559,    # 1.025 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 831723397,   # 1.033 x algorithmic
 }
 
 
@@ -229,6 +231,22 @@ def main():
         out["finalize_avg_us"] = statistics.fmean(fin_us)
     else:
         out["roofline"] = roof(fwd_bytes, fwd_avg, "forward")
+
+    # ---- the same launches back to back (no event between them): each figure is the span of N launches
+    # divided by N, so it holds a launch gap but no end-of-kernel cache write-back forced by an event --
+    def span_us(fn, n=30):
+        for i in range(3):
+            fn(i)
+        ev.record(0, stream)
+        for i in range(n):
+            fn(i)
+        ev.record(1, stream)
+        torch.cuda.synchronize()
+        return ev.elapsed_us(0, 1) / n
+
+    out["back_to_back_us"] = {"forward": span_us(fwd)}
+    if fwd_bwd:
+        out["back_to_back_us"]["backward_plus_finalize"] = span_us(bwd)
 
     # ---- what a plain copy reaches on this box (context for the roofline fraction) ----------------
     cp_us = []
