@@ -117,6 +117,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
+    ap.add_argument("--residual", action="store_true",
+                    help="fused residual variant: y = x + conv(x), dx = dy + conv^T(dy) (same traffic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=65536)
     args = ap.parse_args()
@@ -151,16 +153,17 @@ def main():
     ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     cu, w, b = d.cu_seqlens, d.weight, d.bias
+    flags = _lib.RESIDUAL if args.residual else 0
     def fwd(i):
         j = i % NSET
-        _lib.check(lib.nplm_dwconv_fwd(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(), ys[j].data_ptr(),
-                                       T, C, K, S, act, act, stream), "nplm_dwconv_fwd")
+        _lib.check(lib.nplm_dwconv_fwd_ex(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(),
+                                          ys[j].data_ptr(), T, C, K, S, act, act, flags, stream), "nplm_dwconv_fwd_ex")
 
     def bwd(i, t=None):
         j = i % NSET
         args_ = (xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(),
-                 db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act, stream)
-        rc = lib.nplm_dwconv_bwd(*args_) if t is None else lib.nplm_dwconv_bwd_tuned(*args_, t)
+                 db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act)
+        rc = lib.nplm_dwconv_bwd_ex(*args_, flags, stream) if t is None else lib.nplm_dwconv_bwd_tuned(*args_, stream, t)
         _lib.check(rc, "nplm_dwconv_bwd")
 
     def step(i):
@@ -187,7 +190,7 @@ def main():
     evs = [HipEvents(4) for _ in range(n_ev)]
     tunes = []
     for i in range(n_ev):
-        t = _lib.Tuning()
+        t = _lib.Tuning(flags=flags)
         t.mid_event = evs[i].ev[2]
         tunes.append(t)
     for i in range(n_ev):
@@ -220,7 +223,7 @@ def main():
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
         "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
-                   "rotating_sets": NSET},
+                   "rotating_sets": NSET, "residual": bool(args.residual)},
         "step_algorithmic_bytes": wl.algorithmic_bytes(),
         "step_GBps": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,

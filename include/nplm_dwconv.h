@@ -62,6 +62,10 @@ extern "C" {
 #define NPLM_DWCONV_EALIGN     5  /* activation pointer not aligned to its element size */
 #define NPLM_DWCONV_EWORKSPACE 6  /* workspace NULL, misaligned (256 B) or smaller than required */
 #define NPLM_DWCONV_ECU        7  /* check_cu: cu[0] != 0, cu decreasing, or cu[S] != T */
+#define NPLM_DWCONV_EFLAGS     9  /* unknown bits set in `flags` (8 is used by the internal tuning interface) */
+
+/* flags of the _ex entry points */
+#define NPLM_DWCONV_RESIDUAL 1u   /* fuse the residual connection: y = x + conv(x), dx = dy + conv^T(dy) */
 
 #define NPLM_DWCONV_MAX_K 255
 
@@ -80,6 +84,17 @@ const char* nplm_dwconv_strerror(int code);
 int nplm_dwconv_fwd(const void* x, const int32_t* cu, const void* w, const void* b, void* y,
                     int64_t T, int32_t C, int32_t K, int32_t S,
                     int32_t act_dtype, int32_t w_dtype, void* stream);
+
+/*
+ * Forward with flags. NPLM_DWCONV_RESIDUAL computes y = x + conv(x; w, b): the residual connection
+ * around the module at its call site (x = x + conv(x, cu_seqlens) in the encoder layer,
+ * modeling.py:421-439) without the extra pass over x and y an elementwise add would cost. The centre
+ * tap is valid for every row, so the identity is folded into the centre weight in registers
+ * (exact for bf16 weights; the sum is rounded once). flags == 0 is nplm_dwconv_fwd.
+ */
+int nplm_dwconv_fwd_ex(const void* x, const int32_t* cu, const void* w, const void* b, void* y,
+                       int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
  * Bytes of device workspace nplm_dwconv_bwd needs for these sizes (fp32 partial sums of dw/db,
@@ -101,6 +116,16 @@ int nplm_dwconv_bwd(const void* x, const void* dy, const int32_t* cu, const void
                     void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,
                     int64_t T, int32_t C, int32_t K, int32_t S,
                     int32_t act_dtype, int32_t w_dtype, void* stream);
+
+/*
+ * Backward with flags. With NPLM_DWCONV_RESIDUAL, dx = dy + conv^T(dy; w) (the gradient of
+ * x + conv(x) with respect to x); dw and db are those of the convolution and do not change.
+ * flags == 0 is nplm_dwconv_bwd.
+ */
+int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const void* w,
+                       void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,
+                       int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
  * Debug helper: copies cu to the host (synchronises `stream`) and verifies the preconditions.

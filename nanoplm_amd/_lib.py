@@ -13,14 +13,17 @@ LIB_PATH = os.path.join(_HERE, "libnplm_dwconv.so")
 
 F32 = 0
 BF16 = 1
+RESIDUAL = 1    # NPLM_DWCONV_RESIDUAL
 
 # every symbol include/nplm_dwconv.h declares
 PUBLIC_SYMBOLS = (
     "nplm_dwconv_version",
     "nplm_dwconv_strerror",
     "nplm_dwconv_fwd",
+    "nplm_dwconv_fwd_ex",
     "nplm_dwconv_bwd_workspace_bytes",
     "nplm_dwconv_bwd",
+    "nplm_dwconv_bwd_ex",
     "nplm_dwconv_check_cu",
 )
 
@@ -32,7 +35,7 @@ class Tuning(ctypes.Structure):
 
     _fields_ = [(n, ctypes.c_int32) for n in
                 ("vec", "unroll", "tile_rows", "bw", "bt", "nbt", "xcd_remap", "maxt", "algo", "nwl", "nbuf")
-                ] + [("mid_event", ctypes.c_void_p)]
+                ] + [("flags", ctypes.c_uint32), ("mid_event", ctypes.c_void_p)]
 
 
 def load():
@@ -53,6 +56,8 @@ def load():
     fwd_args = [vp, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32, vp]
     lib.nplm_dwconv_fwd.argtypes = fwd_args
     lib.nplm_dwconv_fwd.restype = ctypes.c_int
+    lib.nplm_dwconv_fwd_ex.argtypes = fwd_args[:-1] + [ctypes.c_uint32, vp]
+    lib.nplm_dwconv_fwd_ex.restype = ctypes.c_int
     lib.nplm_dwconv_fwd_tuned.argtypes = fwd_args + [ctypes.POINTER(Tuning)]
     lib.nplm_dwconv_fwd_tuned.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
@@ -60,6 +65,8 @@ def load():
     bwd_args = [vp, vp, vp, vp, vp, vp, vp, vp, sz, i64, i32, i32, i32, i32, i32, vp]
     lib.nplm_dwconv_bwd.argtypes = bwd_args
     lib.nplm_dwconv_bwd.restype = ctypes.c_int
+    lib.nplm_dwconv_bwd_ex.argtypes = bwd_args[:-1] + [ctypes.c_uint32, vp]
+    lib.nplm_dwconv_bwd_ex.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_tuned.argtypes = bwd_args + [ctypes.POINTER(Tuning)]
     lib.nplm_dwconv_bwd_tuned.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_slabs.argtypes = [i64, i32, i32, i32, ctypes.POINTER(Tuning)]

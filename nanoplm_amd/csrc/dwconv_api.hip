@@ -104,9 +104,9 @@ int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bi
     return 0;
 }
 
-Geo make_geo(const Plan& p, long long T, int C, int S, int w_bf16) {
+Geo make_geo(const Plan& p, long long T, int C, int S, int w_flags) {
     Geo g{};
-    g.T = (int32_t)T; g.C = C; g.S = S; g.w_bf16 = w_bf16;
+    g.T = (int32_t)T; g.C = C; g.S = S; g.w_flags = w_flags;
     g.R = p.R; g.ntiles = p.ntiles; g.ncols = p.ncols; g.nwc = p.nwc;
     g.bw = p.bw; g.bt = p.bt; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_remap = p.remap;
     return g;
@@ -203,9 +203,9 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     return 0;
 }
 
-LdsGeo make_lds_geo(const LdsPlan& p, long long T, int C, int S, int w_bf16) {
+LdsGeo make_lds_geo(const LdsPlan& p, long long T, int C, int S, int w_flags) {
     LdsGeo g{};
-    g.T = (int32_t)T; g.C = C; g.S = S; g.w_bf16 = w_bf16;
+    g.T = (int32_t)T; g.C = C; g.S = S; g.w_flags = w_flags;
     g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_group = p.xcd_group;
     return g;
 }
@@ -266,13 +266,20 @@ hipError_t fill_zero(float* p, long long n, hipStream_t s) {
     return hipGetLastError();
 }
 
+// launch flags of the kernels (W_BF16 | W_RESIDUAL) from the ABI's weight dtype and flags
+int kernel_w_flags(int32_t w_dtype, uint32_t flags) {
+    return (w_dtype == NPLM_DWCONV_BF16 ? W_BF16 : 0) | ((flags & NPLM_DWCONV_RESIDUAL) ? W_RESIDUAL : 0);
+}
+
 int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T, int32_t C,
-             int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
+             int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream,
              const nplm_dwconv_tuning* tune) {
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
     if (T == 0) return 0;
     if (!x || !cu || !w || !y) return -NPLM_DWCONV_ENULL;
+    const int w_flags = kernel_w_flags(w_dtype, flags);
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t E = bf16 ? 2 : 4;
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
@@ -287,7 +294,7 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
         rc = make_lds_plan(false, bf16, T, C, K, tune, &lp);
         if (rc) return rc;
         const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
-        const hipError_t e = launch_fwd_lds(K, lp, la, make_lds_geo(lp, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
+        const hipError_t e = launch_fwd_lds(K, lp, la, make_lds_geo(lp, T, C, S, w_flags), s);
         if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
         return (int)e;
     }
@@ -300,23 +307,25 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
         if (blocks > kNumCU * 16) blocks = kNumCU * 16;
         if (bf16)
             hipLaunchKernelGGL(dwconv_generic_rows_kernel<true>, dim3(blocks), dim3(wpb * 64), 0, s, x, cu, w, b, y,
-                               (int)T, C, S, K, (int)(w_dtype == NPLM_DWCONV_BF16), 0);
+                               (int)T, C, S, K, w_flags, 0);
         else
             hipLaunchKernelGGL(dwconv_generic_rows_kernel<false>, dim3(blocks), dim3(wpb * 64), 0, s, x, cu, w, b, y,
-                               (int)T, C, S, K, (int)(w_dtype == NPLM_DWCONV_BF16), 0);
+                               (int)T, C, S, K, w_flags, 0);
         return (int)hipGetLastError();
     }
     const ConvPtrs a{x, nullptr, cu, w, b, y, nullptr};
-    const hipError_t e = launch_fwd(K, bf16, p, a, make_geo(p, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
+    const hipError_t e = launch_fwd(K, bf16, p, a, make_geo(p, T, C, S, w_flags), s);
     if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
     return (int)e;
 }
 
 int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw, float* db,
              void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K, int32_t S,
-             int32_t act_dtype, int32_t w_dtype, void* stream, const nplm_dwconv_tuning* tune) {
+             int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream, const nplm_dwconv_tuning* tune) {
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    const int w_flags = kernel_w_flags(w_dtype, flags);
     hipStream_t s = (hipStream_t)stream;
     const bool want_red = dw || db;
     if (T == 0) {
@@ -348,7 +357,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         }
         const ConvPtrs la{x, dy, cu, w, nullptr, dx, part};
         hipError_t e = launch_bwd_lds(K, lp, dx != nullptr, want_red, la,
-                                      make_lds_geo(lp, T, C, S, w_dtype == NPLM_DWCONV_BF16), s);
+                                      make_lds_geo(lp, T, C, S, w_flags), s);
         if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
         if (e != hipSuccess) return (int)e;
         if (tune && tune->mid_event) {
@@ -383,7 +392,6 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
             return -NPLM_DWCONV_EWORKSPACE;
         partial = reinterpret_cast<float*>(workspace);
     }
-    const int w_bf16 = (w_dtype == NPLM_DWCONV_BF16);
 
     if (p.generic) {
         if (dx) {
@@ -392,10 +400,10 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
             if (blocks > kNumCU * 16) blocks = kNumCU * 16;
             if (bf16)
                 hipLaunchKernelGGL(dwconv_generic_rows_kernel<true>, dim3(blocks), dim3(wpb * 64), 0, s, dy, cu, w,
-                                   (const void*)nullptr, dx, (int)T, C, S, K, w_bf16, 1);
+                                   (const void*)nullptr, dx, (int)T, C, S, K, w_flags, 1);
             else
                 hipLaunchKernelGGL(dwconv_generic_rows_kernel<false>, dim3(blocks), dim3(wpb * 64), 0, s, dy, cu, w,
-                                   (const void*)nullptr, dx, (int)T, C, S, K, w_bf16, 1);
+                                   (const void*)nullptr, dx, (int)T, C, S, K, w_flags, 1);
             const hipError_t e = hipGetLastError();
             if (e != hipSuccess) return (int)e;
         }
@@ -413,7 +421,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         }
     } else {
         const ConvPtrs a{x, dy, cu, w, nullptr, dx, partial};
-        const hipError_t e = launch_bwd(K, bf16, p, dx != nullptr, want_red, a, make_geo(p, T, C, S, w_bf16), s);
+        const hipError_t e = launch_bwd(K, bf16, p, dx != nullptr, want_red, a, make_geo(p, T, C, S, w_flags), s);
         if (e == hipErrorInvalidConfiguration && tune) return -NPLM_DWCONV_ETUNING;
         if (e != hipSuccess) return (int)e;
     }
@@ -451,6 +459,7 @@ const char* nplm_dwconv_strerror(int code) {
         case NPLM_DWCONV_EALIGN: return "nplm_dwconv: pointer not aligned to its element size";
         case NPLM_DWCONV_EWORKSPACE: return "nplm_dwconv: workspace NULL, not 256-byte aligned, or too small";
         case NPLM_DWCONV_ECU: return "nplm_dwconv: cu_seqlens must start at 0, be non-decreasing and end at T";
+        case NPLM_DWCONV_EFLAGS: return "nplm_dwconv: unknown bits set in flags";
         case NPLM_DWCONV_ETUNING: return "nplm_dwconv: geometry override not available in this build";
     }
     return "nplm_dwconv: unknown error code";
@@ -458,13 +467,18 @@ const char* nplm_dwconv_strerror(int code) {
 
 int nplm_dwconv_fwd(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T, int32_t C,
                     int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream) {
-    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, stream, nullptr);
+    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, 0, stream, nullptr);
+}
+
+int nplm_dwconv_fwd_ex(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T, int32_t C,
+                       int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
+    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, flags, stream, nullptr);
 }
 
 int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const void* b, void* y, int64_t T,
                           int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
                           const nplm_dwconv_tuning* tune) {
-    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, stream, tune);
+    return fwd_impl(x, cu, w, b, y, T, C, K, S, act_dtype, w_dtype, tune ? tune->flags : 0u, stream, tune);
 }
 
 size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
@@ -501,16 +515,23 @@ int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype
 int nplm_dwconv_bwd(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw, float* db,
                     void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K, int32_t S,
                     int32_t act_dtype, int32_t w_dtype, void* stream) {
-    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, stream,
+    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, 0, stream,
                     nullptr);
+}
+
+int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw, float* db,
+                       void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
+    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, flags,
+                    stream, nullptr);
 }
 
 int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw,
                           float* db, void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K,
                           int32_t S, int32_t act_dtype, int32_t w_dtype, void* stream,
                           const nplm_dwconv_tuning* tune) {
-    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, stream,
-                    tune);
+    return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype,
+                    tune ? tune->flags : 0u, stream, tune);
 }
 
 int nplm_dwconv_debug_copy(const void* src, void* dst, size_t bytes, void* stream) {

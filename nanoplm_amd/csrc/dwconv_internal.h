@@ -25,6 +25,7 @@ typedef struct nplm_dwconv_tuning {
     int32_t algo;       // 1 = sliding-window (register) kernels, 2 = LDS-staged pipelined kernels
     int32_t nwl;        // LDS kernels: loader waves per block
     int32_t nbuf;       // LDS forward: tile buffers (2 or 3)
+    uint32_t flags;     // NPLM_DWCONV_RESIDUAL etc., as for the _ex entry points
     void* mid_event;    // backward: hipEvent_t recorded between the fused kernel and the finalize kernel
 } nplm_dwconv_tuning;
 // For algo 2 the fields mean: vec = channels per lane, unroll = rows per wave (RW), bt = row groups

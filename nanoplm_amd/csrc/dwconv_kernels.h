@@ -33,7 +33,7 @@ namespace nplm {
 // __restrict__ kernel arguments so that cu is read through the scalar data path.
 struct Geo {
     int32_t T, C, S;
-    int32_t w_bf16;
+    int32_t w_flags;       // W_BF16: weights/bias are bf16 (else fp32); W_RESIDUAL: the identity is added (see load_weights)
     int32_t R;             // rows per tile (multiple of U)
     int32_t ntiles;        // ceil(T / R)
     int32_t ncols;         // C / VEC
@@ -58,9 +58,16 @@ __device__ __forceinline__ void block_coords(const Geo& g, int& cb, int& tb) {
     tb = b / g.ncb;
 }
 
+// Bits of the w_flags launch parameter.
+constexpr int W_BF16 = 1;      // weights and bias are bf16 (otherwise fp32)
+constexpr int W_RESIDUAL = 2;  // compute x + conv(x) (forward) / dy + conv^T(dy) (dx)
+
+// Weights of channels c0 .. c0+VEC-1 as fp32 registers. The fused residual costs nothing: the centre
+// tap is valid for every row, so x + conv(x; w) = conv(x; w + delta_centre); one is added to the
+// centre weight here (exact for bf16 weights, one fp32 rounding otherwise). dw does not read wr.
 template <int VEC, int K>
-__device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_bf16, int c0, float (&wr)[VEC][K]) {
-    if (w_bf16) {
+__device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_flags, int c0, float (&wr)[VEC][K]) {
+    if (w_flags & W_BF16) {
         const uint16_t* wp = reinterpret_cast<const uint16_t*>(w) + (size_t)c0 * K;
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
@@ -72,6 +79,10 @@ __device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_b
         for (int v = 0; v < VEC; ++v)
 #pragma unroll
             for (int k = 0; k < K; ++k) wr[v][k] = wp[v * K + k];
+    }
+    if (w_flags & W_RESIDUAL) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) wr[v][(K - 1) / 2] += 1.f;
     }
 }
 
@@ -131,14 +142,14 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
     const int T = g.T, S = g.S, R = g.R;
 
     float wr[VEC][K];
-    load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+    load_weights<VEC, K>(w, g.w_flags, c0, wr);
     float bias[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
     if (b) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
-            bias[v] = g.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
+            bias[v] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
                                : reinterpret_cast<const float*>(b)[c0 + v];
     }
 
@@ -278,7 +289,7 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
     const int T = g.T, S = g.S, R = g.R;
 
     float wr[VEC][K];
-    if constexpr (WDX) load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+    if constexpr (WDX) load_weights<VEC, K>(w, g.w_flags, c0, wr);
     float dwa[VEC][K];
     float dba[VEC];
 #pragma unroll
@@ -493,8 +504,8 @@ __device__ __forceinline__ void st_act(void* p, size_t i, float f) {
     if constexpr (BF16) reinterpret_cast<uint16_t*>(p)[i] = f32_to_bf16(f);
     else reinterpret_cast<float*>(p)[i] = f;
 }
-__device__ __forceinline__ float ld_w(const void* p, int w_bf16, size_t i) {
-    return w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p)[i]) : reinterpret_cast<const float*>(p)[i];
+__device__ __forceinline__ float ld_w(const void* p, int w_flags, size_t i) {
+    return (w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(p)[i]) : reinterpret_cast<const float*>(p)[i];
 }
 
 // flip = 0: out[t] = b + sum_k w[k] * in[t+k-P]   (forward)
@@ -502,7 +513,7 @@ __device__ __forceinline__ float ld_w(const void* p, int w_bf16, size_t i) {
 template <bool BF16>
 __global__ void dwconv_generic_rows_kernel(const void* in, const int32_t* __restrict__ cu, const void* w,
                                            const void* b, void* out, int T, int C, int S, int K,
-                                           int w_bf16, int flip) {
+                                           int w_flags, int flip) {
     const int P = (K - 1) / 2;
     const int lane = (int)(threadIdx.x & 63);
     const int wpb = (int)(blockDim.x >> 6);
@@ -513,12 +524,15 @@ __global__ void dwconv_generic_rows_kernel(const void* in, const int32_t* __rest
     for (int t = gw; t < T; t += nw) {
         sc.locate(cu, S, T, t, sc.seq);
         for (int c = lane; c < C; c += 64) {
-            float acc = (b && !flip) ? ld_w(b, w_bf16, c) : 0.f;
+            float acc = (b && !flip) ? ld_w(b, w_flags, c) : 0.f;
             for (int k = 0; k < K; ++k) {
                 const int j = flip ? (t - k + P) : (t + k - P);
                 // cu only masks; the explicit [0, T) test keeps a malformed cu from forming a bad address
-                if (j >= sc.cs && j < sc.ce && j >= 0 && j < T)
-                    acc = __builtin_fmaf(ld_w(w, w_bf16, (size_t)c * K + k), ld_act<BF16>(in, (size_t)j * C + c), acc);
+                if (j >= sc.cs && j < sc.ce && j >= 0 && j < T) {
+                    float wk = ld_w(w, w_flags, (size_t)c * K + k);
+                    if (k == P && (w_flags & W_RESIDUAL)) wk += 1.f;
+                    acc = __builtin_fmaf(wk, ld_act<BF16>(in, (size_t)j * C + c), acc);
+                }
             }
             st_act<BF16>(out, (size_t)t * C + c, acc);
         }

@@ -41,7 +41,7 @@ namespace nplm {
 
 struct LdsGeo {
     int32_t T, C, S;
-    int32_t w_bf16;
+    int32_t w_flags;    // W_BF16 | W_RESIDUAL
     int32_t ntiles;     // ceil(T / R)
     int32_t ncb, nbt;   // grid = ncb column blocks x nbt token blocks (nbt <= ntiles)
     int32_t xcd_group;  // > 0: runs of this many adjacent token-blocks share an XCD (and its L2)
@@ -263,11 +263,11 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
             wait_vmem_all();
         }
     } else {
-        load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+        load_weights<VEC, K>(w, g.w_flags, c0, wr);
         if (b) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
-                bias[v] = g.w_bf16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
+                bias[v] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
                                    : reinterpret_cast<const float*>(b)[c0 + v];
         }
     }
@@ -418,7 +418,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         stage_both(lds_raw, tb * R);
         wait_vmem_all();
     } else {
-        if constexpr (WDX) load_weights<VEC, K>(w, g.w_bf16, c0, wr);
+        if constexpr (WDX) load_weights<VEC, K>(w, g.w_flags, c0, wr);
     }
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;

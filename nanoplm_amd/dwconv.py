@@ -7,6 +7,10 @@ Drop-in surface for the conv on the packed path of the encoder layer
     y = VarlenDWConv1dFunction.apply(x, cu_seqlens, weight, bias)
     conv = VarlenDWConv1d(channels=C, kernel_size=K);  y = conv(x, cu_seqlens)
 
+``residual=True`` (function argument / module option) fuses the residual connection a caller would
+write as ``x = x + conv(x, cu_seqlens)``: the kernels compute ``x + conv(x)`` and ``dy + conv^T(dy)``
+directly, which saves the elementwise add's three passes over [T, C] in each direction.
+
 All arithmetic runs in hand-written HIP kernels reached through the C ABI of libnplm_dwconv.so.
 There is deliberately no CPU or pure-PyTorch implementation here: tensors that are not on a ROCm
 device, or a missing shared library, raise.
@@ -55,8 +59,15 @@ def _validate(x, cu_seqlens, weight, bias):
     return T, C, K, cu_seqlens.numel() - 1
 
 
-def varlen_dwconv_fwd(x, cu_seqlens, weight, bias=None, *, tuning: Optional[_lib.Tuning] = None):
-    """y = conv(x) (same dtype as x). Raw forward without autograd."""
+def _with_flags(tuning: _lib.Tuning, flags: int) -> _lib.Tuning:
+    t = _lib.Tuning.from_buffer_copy(tuning)
+    t.flags = flags
+    return t
+
+
+def varlen_dwconv_fwd(x, cu_seqlens, weight, bias=None, *, residual: bool = False,
+                      tuning: Optional[_lib.Tuning] = None):
+    """y = conv(x), or x + conv(x) with ``residual`` (same dtype as x). Raw forward without autograd."""
     T, C, K, S = _validate(x, cu_seqlens, weight, bias)
     lib = _lib.load()
     x = x.contiguous()
@@ -67,12 +78,13 @@ def varlen_dwconv_fwd(x, cu_seqlens, weight, bias=None, *, tuning: Optional[_lib
     y = torch.empty_like(x)
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream().cuda_stream
+        flags = _lib.RESIDUAL if residual else 0
         args = (_ptr(x), _ptr(cu_seqlens), _ptr(weight), _ptr(bias), _ptr(y), T, C, K, S,
-                _DTYPES[x.dtype], _DTYPES[weight.dtype], stream)
+                _DTYPES[x.dtype], _DTYPES[weight.dtype])
         if tuning is None:
-            rc = lib.nplm_dwconv_fwd(*args)
+            rc = lib.nplm_dwconv_fwd_ex(*args, flags, stream)
         else:
-            rc = lib.nplm_dwconv_fwd_tuned(*args, tuning)
+            rc = lib.nplm_dwconv_fwd_tuned(*args, stream, _with_flags(tuning, flags))
     _lib.check(rc, "nplm_dwconv_fwd")
     return y
 
@@ -82,9 +94,11 @@ def bwd_workspace_bytes(T: int, C: int, K: int, dtype: torch.dtype) -> int:
     return int(_lib.load().nplm_dwconv_bwd_workspace_bytes(T, C, K, _DTYPES[dtype]))
 
 
-def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True,
+def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, residual: bool = False,
                       tuning: Optional[_lib.Tuning] = None, workspace: Optional[torch.Tensor] = None):
-    """(dx, dw, db): dx in x's dtype (or None), dw [C,K] and db [C] in fp32 (or None, None)."""
+    """(dx, dw, db): dx in x's dtype (or None), dw [C,K] and db [C] in fp32 (or None, None).
+
+    With ``residual`` dx is the gradient of x + conv(x), i.e. dy + conv^T(dy); dw and db do not change."""
     T, C, K, S = _validate(x, cu_seqlens, weight, None)
     if dy.shape != x.shape or dy.dtype != x.dtype or dy.device != x.device:
         raise ValueError("dy must match x in shape, dtype and device")
@@ -105,13 +119,14 @@ def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True,
                 nbytes = int(lib.nplm_dwconv_bwd_slabs(T, C, K, act, tuning)) * (K + 1) * C * 4
             workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
         stream = torch.cuda.current_stream().cuda_stream
+        flags = _lib.RESIDUAL if residual else 0
         args = (_ptr(x), _ptr(dy), _ptr(cu_seqlens), _ptr(weight), _ptr(dx), _ptr(dw), _ptr(db),
                 _ptr(workspace), 0 if workspace is None else workspace.numel() * workspace.element_size(),
-                T, C, K, S, act, _DTYPES[weight.dtype], stream)
+                T, C, K, S, act, _DTYPES[weight.dtype])
         if tuning is None:
-            rc = lib.nplm_dwconv_bwd(*args)
+            rc = lib.nplm_dwconv_bwd_ex(*args, flags, stream)
         else:
-            rc = lib.nplm_dwconv_bwd_tuned(*args, tuning)
+            rc = lib.nplm_dwconv_bwd_tuned(*args, stream, _with_flags(tuning, flags))
     _lib.check(rc, "nplm_dwconv_bwd")
     return dx, dw, db
 
@@ -128,7 +143,7 @@ def check_cu_seqlens(cu_seqlens: torch.Tensor, T: int) -> None:
 
 
 class VarlenDWConv1dFunction(torch.autograd.Function):
-    """``apply(x, cu_seqlens, weight, bias) -> y``; backward returns ``(dx, None, dw, db)``.
+    """``apply(x, cu_seqlens, weight, bias[, residual]) -> y``; backward returns ``(dx, None, dw, db[, None])``.
 
     dw and db are reduced and produced in fp32 by the kernels and cast to the parameters' dtypes
     only here. Under ``torch.autocast`` the op takes its inputs as they come (bf16 activations
@@ -136,10 +151,11 @@ class VarlenDWConv1dFunction(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, x, cu_seqlens, weight, bias=None):
-        y = varlen_dwconv_fwd(x, cu_seqlens, weight, bias)
+    def forward(ctx, x, cu_seqlens, weight, bias=None, residual=False):
+        y = varlen_dwconv_fwd(x, cu_seqlens, weight, bias, residual=bool(residual))
         ctx.save_for_backward(x, cu_seqlens, weight)
         ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.residual = bool(residual)
         return y
 
     @staticmethod
@@ -149,16 +165,17 @@ class VarlenDWConv1dFunction(torch.autograd.Function):
         need_dw = ctx.needs_input_grad[2] or (ctx.bias_dtype is not None and ctx.needs_input_grad[3])
         if dy.dtype != x.dtype:
             dy = dy.to(x.dtype)
-        dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, need_dx=need_dx, need_dw=need_dw)
+        dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, need_dx=need_dx, need_dw=need_dw,
+                                       residual=ctx.residual)
         if dw is not None:
             dw = dw.to(weight.dtype) if ctx.needs_input_grad[2] else None
             db = db.to(ctx.bias_dtype) if (ctx.bias_dtype is not None and ctx.needs_input_grad[3]) else None
-        return dx, None, dw, db
+        return dx, None, dw, db, None
 
 
-def varlen_dwconv(x, cu_seqlens, weight, bias=None):
+def varlen_dwconv(x, cu_seqlens, weight, bias=None, residual: bool = False):
     """Functional form of :class:`VarlenDWConv1dFunction`."""
-    return VarlenDWConv1dFunction.apply(x, cu_seqlens, weight, bias)
+    return VarlenDWConv1dFunction.apply(x, cu_seqlens, weight, bias, residual)
 
 
 class VarlenDWConv1d(nn.Module):
@@ -166,14 +183,17 @@ class VarlenDWConv1d(nn.Module):
 
     ``weight`` is ``[C, K]`` (tap k multiplies row ``t + k - (K-1)//2``), ``bias`` is ``[C]``.
     Rows outside a sequence read as zero; nothing crosses a sequence boundary.
+    ``residual=True`` makes the module return ``x + conv(x)`` from the same single pass.
     """
 
-    def __init__(self, channels: int, kernel_size: int, bias: bool = True, device=None, dtype=None):
+    def __init__(self, channels: int, kernel_size: int, bias: bool = True, residual: bool = False,
+                 device=None, dtype=None):
         super().__init__()
         if kernel_size < 1 or kernel_size % 2 == 0:
             raise ValueError(f"kernel_size must be odd and positive, got {kernel_size}")
         self.channels = channels
         self.kernel_size = kernel_size
+        self.residual = bool(residual)
         self.weight = nn.Parameter(torch.empty((channels, kernel_size), device=device, dtype=dtype))
         self.bias = nn.Parameter(torch.empty((channels,), device=device, dtype=dtype)) if bias else None
         self.reset_parameters()
@@ -187,11 +207,12 @@ class VarlenDWConv1d(nn.Module):
     def forward(self, x: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
         if torch.compiler.is_compiling():
             # under torch.compile the opaque custom ops keep the graph whole
-            return varlen_dwconv_fwd_op(x, cu_seqlens, self.weight, self.bias)
-        return VarlenDWConv1dFunction.apply(x, cu_seqlens, self.weight, self.bias)
+            return varlen_dwconv_fwd_op(x, cu_seqlens, self.weight, self.bias, self.residual)
+        return VarlenDWConv1dFunction.apply(x, cu_seqlens, self.weight, self.bias, self.residual)
 
     def extra_repr(self) -> str:
-        return f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}"
+        return (f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}, "
+                f"residual={self.residual}")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -202,47 +223,48 @@ class VarlenDWConv1d(nn.Module):
 # ---------------------------------------------------------------------------------------------
 @torch.library.custom_op("nanoplm_amd::varlen_dwconv_fwd", mutates_args=(), device_types="cuda")
 def varlen_dwconv_fwd_op(x: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
-                         bias: Optional[torch.Tensor]) -> torch.Tensor:
-    return varlen_dwconv_fwd(x, cu_seqlens, weight, bias)
+                         bias: Optional[torch.Tensor], residual: bool = False) -> torch.Tensor:
+    return varlen_dwconv_fwd(x, cu_seqlens, weight, bias, residual=residual)
 
 
 @varlen_dwconv_fwd_op.register_fake
-def _(x, cu_seqlens, weight, bias):
+def _(x, cu_seqlens, weight, bias, residual=False):
     return torch.empty_like(x, memory_format=torch.contiguous_format)
 
 
 @torch.library.custom_op("nanoplm_amd::varlen_dwconv_bwd", mutates_args=(), device_types="cuda")
-def varlen_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor,
-                         weight: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+def varlen_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
+                         residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dx, dw, db) with dw [C,K] and db [C] in fp32."""
-    dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight)
+    dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, residual=residual)
     return dx, dw, db
 
 
 @varlen_dwconv_bwd_op.register_fake
-def _(x, dy, cu_seqlens, weight):
+def _(x, dy, cu_seqlens, weight, residual=False):
     C, K = weight.shape
     return (torch.empty_like(x, memory_format=torch.contiguous_format),
             x.new_empty((C, K), dtype=torch.float32), x.new_empty((C,), dtype=torch.float32))
 
 
 def _op_setup_context(ctx, inputs, output):
-    x, cu_seqlens, weight, bias = inputs
+    x, cu_seqlens, weight, bias, residual = inputs
     ctx.save_for_backward(x, cu_seqlens, weight)
     ctx.bias_dtype = None if bias is None else bias.dtype
+    ctx.residual = bool(residual)
 
 
 def _op_backward(ctx, dy):
     x, cu_seqlens, weight = ctx.saved_tensors
     if dy.dtype != x.dtype:
         dy = dy.to(x.dtype)
-    dx, dw, db = varlen_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, weight)
-    return dx, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype))
+    dx, dw, db = varlen_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, weight, ctx.residual)
+    return dx, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype)), None
 
 
 varlen_dwconv_fwd_op.register_autograd(_op_backward, setup_context=_op_setup_context)
 
 
-def varlen_dwconv_compilable(x, cu_seqlens, weight, bias=None):
+def varlen_dwconv_compilable(x, cu_seqlens, weight, bias=None, residual: bool = False):
     """Same result as :func:`varlen_dwconv`, routed through the registered custom ops (traceable)."""
-    return varlen_dwconv_fwd_op(x, cu_seqlens, weight, bias)
+    return varlen_dwconv_fwd_op(x, cu_seqlens, weight, bias, residual)

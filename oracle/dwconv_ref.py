@@ -35,8 +35,11 @@ _c_lib = None
 # --------------------------------------------------------------------------------------------
 # reference path: per-sequence F.conv1d
 # --------------------------------------------------------------------------------------------
-def ref_dwconv_varlen(x, cu_seqlens, weight, bias=None, compute_dtype=torch.float32):
-    """y[T, C] of the per-sequence conv1d loop, computed in ``compute_dtype`` on x's device."""
+def ref_dwconv_varlen(x, cu_seqlens, weight, bias=None, compute_dtype=torch.float32, residual=False):
+    """y[T, C] of the per-sequence conv1d loop, computed in ``compute_dtype`` on x's device.
+
+    ``residual``: the caller-side residual connection ``x + conv(x)`` written as a separate add, the
+    way an encoder layer applies its sub-modules (modeling.py:421-439)."""
     T, C = x.shape
     K = weight.shape[1]
     assert K % 2 == 1, "same-length output needs an odd kernel size"
@@ -54,15 +57,16 @@ def ref_dwconv_varlen(x, cu_seqlens, weight, bias=None, compute_dtype=torch.floa
         outs.append(ys[0].transpose(0, 1))
     if not outs:
         return xw.new_zeros((0, C))
-    return torch.cat(outs, dim=0)
+    y = torch.cat(outs, dim=0)
+    return xw + y if residual else y
 
 
-def ref_dwconv_varlen_grads(x, cu_seqlens, weight, bias, dy, compute_dtype=torch.float32):
+def ref_dwconv_varlen_grads(x, cu_seqlens, weight, bias, dy, compute_dtype=torch.float32, residual=False):
     """(y, dx, dw, db) of the reference path via autograd, all in ``compute_dtype``."""
     xr = x.detach().to(compute_dtype).requires_grad_(True)
     wr = weight.detach().to(compute_dtype).requires_grad_(True)
     br = None if bias is None else bias.detach().to(compute_dtype).requires_grad_(True)
-    y = ref_dwconv_varlen(xr, cu_seqlens, wr, br, compute_dtype)
+    y = ref_dwconv_varlen(xr, cu_seqlens, wr, br, compute_dtype, residual)
     y.backward(dy.to(compute_dtype))
     db = None if br is None else br.grad
     return y.detach(), xr.grad, wr.grad, db
@@ -104,8 +108,9 @@ def _ptr(a, ct):
     return None if a is None else a.ctypes.data_as(ctypes.POINTER(ct))
 
 
-def c_oracle_fwd(x, cu_seqlens, weight, bias=None):
-    """float64 y[T, C] (torch, CPU) from the C restatement; inputs are upcast to fp32 first."""
+def c_oracle_fwd(x, cu_seqlens, weight, bias=None, residual=False):
+    """float64 y[T, C] (torch, CPU) from the C restatement; inputs are upcast to fp32 first.
+    ``residual`` adds x (in float64) to the result."""
     lib = _load_c()
     xa, wa = _f32(x), _f32(weight)
     ba = None if bias is None else _f32(bias)
@@ -117,11 +122,13 @@ def c_oracle_fwd(x, cu_seqlens, weight, bias=None):
                                     _ptr(ba, ctypes.c_float), _ptr(y, ctypes.c_double), T, C, K, len(cua) - 1)
     if rc:
         raise ValueError("C oracle rejected its inputs (cu_seqlens malformed or K even)")
+    if residual:
+        y += xa
     return torch.from_numpy(y)
 
 
-def c_oracle_bwd(x, dy, cu_seqlens, weight):
-    """float64 (dx[T,C], dw[C,K], db[C]) from the C restatement."""
+def c_oracle_bwd(x, dy, cu_seqlens, weight, residual=False):
+    """float64 (dx[T,C], dw[C,K], db[C]) from the C restatement; ``residual`` adds dy to dx."""
     lib = _load_c()
     xa, ga, wa = _f32(x), _f32(dy), _f32(weight)
     cua = np.ascontiguousarray(cu_seqlens.detach().cpu().numpy().astype(np.int32))
@@ -135,6 +142,8 @@ def c_oracle_bwd(x, dy, cu_seqlens, weight):
                                     _ptr(db, ctypes.c_double), T, C, K, len(cua) - 1)
     if rc:
         raise ValueError("C oracle rejected its inputs (cu_seqlens malformed or K even)")
+    if residual:
+        dx += ga
     return torch.from_numpy(dx), torch.from_numpy(dw), torch.from_numpy(db)
 
 

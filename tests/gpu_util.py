@@ -34,7 +34,7 @@ def assert_act_close(got, ref64, dtype, what):
         scale = float(ref64.abs().max())
         rel = float(err.max()) / max(scale, 1e-30)
         assert rel <= F32_RTOL, f"{what}: max error / max|ref| = {rel:.3e} > {F32_RTOL}"
-        big = ref64.abs() > 1e-3
+        big = ref64.abs() > 1e-2      # below that, cancellation among K terms of size ~1 dominates
         if big.any():
             relel = float((err[big] / ref64[big].abs()).max())
             assert relel <= 2e-4, f"{what}: element-wise relative error {relel:.3e}"

@@ -263,3 +263,39 @@ def test_golden_cfg1_is_configuration_1(golden_dir):
     assert z["x"].shape[1] == 64 and z["w"].shape == (64, 3) and len(z["cu_seqlens"]) == 9
     lens = np.diff(z["cu_seqlens"])
     assert lens.min() >= 20 and lens.max() <= 128
+
+
+# ---- residual connection (x + conv(x)) ---------------------------------------------------------------
+def test_residual_oracles_agree_and_reduce_to_the_centre_weight_identity():
+    """x + conv(x; w) = conv(x; w + delta_centre) because the centre tap is valid for every row; the
+    three statements of the operator agree on it, and the gradients are dy + conv^T(dy), dw, db."""
+    g = torch.Generator().manual_seed(77)
+    lens = torch.tensor([1, 2, 9, 0, 3, 30, 1])
+    cu = torch.zeros(len(lens) + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(lens, 0)
+    T, C, K = int(lens.sum()), 6, 5
+    x = torch.randn(T, C, generator=g, dtype=torch.float64)
+    w = torch.randn(C, K, generator=g, dtype=torch.float64)
+    b = torch.randn(C, generator=g, dtype=torch.float64)
+    dy = torch.randn(T, C, generator=g, dtype=torch.float64)
+    w1 = w.clone()
+    w1[:, (K - 1) // 2] += 1.0
+    y_res, dx_res, dw_res, db_res = O.ref_dwconv_varlen_grads(x, cu, w, b, dy, torch.float64, residual=True)
+    y_id, dx_id, dw_id, db_id = O.ref_dwconv_varlen_grads(x, cu, w1, b, dy, torch.float64)
+    torch.testing.assert_close(y_res, y_id, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dx_res, dx_id, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dw_res, dw_id, rtol=0, atol=1e-12)      # dw does not see the identity
+    torch.testing.assert_close(db_res, db_id, rtol=0, atol=1e-12)
+    yb, dxb, dwb, dbb = O.brute_force(x, cu, w1, b, dy)
+    torch.testing.assert_close(y_res, yb, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dx_res, dxb, rtol=0, atol=1e-12)
+    yc = O.c_oracle_fwd(x.float(), cu, w.float(), b.float(), residual=True)
+    dxc, dwc, dbc = O.c_oracle_bwd(x.float(), dy.float(), cu, w.float(), residual=True)
+    y32, dx32, dw32, db32 = O.ref_dwconv_varlen_grads(x.float(), cu, w.float(), b.float(), dy.float(), torch.float64,
+                                                      residual=True)
+    torch.testing.assert_close(yc, y32, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dxc, dx32, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dwc, dw32, rtol=0, atol=1e-12)
+    # w = 0, b = 0: the identity
+    y0 = O.ref_dwconv_varlen(x, cu, torch.zeros_like(w), None, torch.float64, residual=True)
+    assert torch.equal(y0, x)
