@@ -11,5 +11,13 @@ from .dwconv import (  # noqa: F401
     varlen_dwconv_fwd,
     varlen_dwconv_fwd_op,
 )
+from .padded import (  # noqa: F401
+    is_right_padded,
+    pad_output,
+    padded_dwconv,
+    right_padded_cu_seqlens,
+    unpad_input,
+)
+from .hygiene import conv_parameters, split_conv_parameters  # noqa: F401
 
 __version__ = "0.1.0"

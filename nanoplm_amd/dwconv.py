@@ -184,25 +184,67 @@ class VarlenDWConv1d(nn.Module):
     ``weight`` is ``[C, K]`` (tap k multiplies row ``t + k - (K-1)//2``), ``bias`` is ``[C]``.
     Rows outside a sequence read as zero; nothing crosses a sequence boundary.
     ``residual=True`` makes the module return ``x + conv(x)`` from the same single pass.
+
+    How the parameters meet the reference's training loop:
+
+    * ``flat_weight=True`` registers the taps as a 1-D parameter ``weight_flat`` of ``C*K`` elements
+      (``.weight`` stays available as its ``[C, K]`` view). A 2-D ``[C, K]`` parameter would be routed
+      to Muon by ``build_muon_optimizer`` (src/nanoplm/pretraining/optim.py:43-51 sends every
+      ``ndim == 2`` hidden parameter there; orthogonalising a C x 7 tap table is meaningless) and
+      weight-decayed by ``_use_weight_decay`` (src/nanoplm/pretraining/pure_pipeline.py:68-76);
+      a 1-D parameter lands in the AdamW no-decay group of both, with no change to the reference.
+    * ``init``: ``"normal"`` = N(0, 1/K) taps and N(0, 0.02^2) bias (the benchmark's distributions);
+      ``"zero"`` = all zeros, so a ``residual=True`` block starts as the identity, matching the
+      reference's zero-initialised output projections (modeling.py:602-605); ``"identity"`` = centre
+      tap 1, for the non-residual form. The reference's ``init_weights`` (modeling.py:581-623) has no
+      branch that would touch this module, so the module initialises itself.
     """
 
     def __init__(self, channels: int, kernel_size: int, bias: bool = True, residual: bool = False,
-                 device=None, dtype=None):
+                 flat_weight: bool = False, init: str = "normal", device=None, dtype=None):
         super().__init__()
         if kernel_size < 1 or kernel_size % 2 == 0:
             raise ValueError(f"kernel_size must be odd and positive, got {kernel_size}")
+        if init not in ("normal", "zero", "identity"):
+            raise ValueError(f"init must be 'normal', 'zero' or 'identity', got {init!r}")
         self.channels = channels
         self.kernel_size = kernel_size
         self.residual = bool(residual)
-        self.weight = nn.Parameter(torch.empty((channels, kernel_size), device=device, dtype=dtype))
+        self.flat_weight = bool(flat_weight)
+        self.init = init
+        if self.flat_weight:
+            self.weight_flat = nn.Parameter(torch.empty((channels * kernel_size,), device=device, dtype=dtype))
+        else:
+            self.weight = nn.Parameter(torch.empty((channels, kernel_size), device=device, dtype=dtype))
         self.bias = nn.Parameter(torch.empty((channels,), device=device, dtype=dtype)) if bias else None
         self.reset_parameters()
 
+    def __getattr__(self, name):
+        # .weight of a flat_weight module: the [C, K] view of the 1-D parameter (autograd flows through it)
+        if name == "weight" and "weight_flat" in self.__dict__.get("_parameters", {}):
+            return self._parameters["weight_flat"].view(self.channels, self.kernel_size)
+        return super().__getattr__(name)
+
+    @torch.no_grad()
     def reset_parameters(self) -> None:
-        # variance 1/K per tap, small bias: the distributions the benchmark configs draw from
-        nn.init.normal_(self.weight, mean=0.0, std=1.0 / math.sqrt(self.kernel_size))
+        w = self.weight
+        if self.init == "normal":
+            nn.init.normal_(w, mean=0.0, std=1.0 / math.sqrt(self.kernel_size))
+        else:
+            w.zero_()
+            if self.init == "identity":
+                w[:, (self.kernel_size - 1) // 2] = 1.0
         if self.bias is not None:
-            nn.init.normal_(self.bias, mean=0.0, std=0.02)
+            if self.init == "normal":
+                nn.init.normal_(self.bias, mean=0.0, std=0.02)
+            else:
+                self.bias.zero_()
+
+    def forward_padded(self, x: torch.Tensor, attention_mask: torch.Tensor,
+                       assume_right_padded: bool = True) -> torch.Tensor:
+        """Padded-batch door: ``x:[B, L, C]``, ``attention_mask:[B, L]`` (see nanoplm_amd.padded)."""
+        from .padded import padded_dwconv
+        return padded_dwconv(x, attention_mask, self.weight, self.bias, self.residual, assume_right_padded)
 
     def forward(self, x: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
         if torch.compiler.is_compiling():
@@ -212,7 +254,7 @@ class VarlenDWConv1d(nn.Module):
 
     def extra_repr(self) -> str:
         return (f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}, "
-                f"residual={self.residual}")
+                f"residual={self.residual}, flat_weight={self.flat_weight}, init={self.init}")
 
 
 # ---------------------------------------------------------------------------------------------
