@@ -170,7 +170,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    p.sh = lds_default_shape(bwd, bf16);
+    p.sh = lds_default_shape(bwd, bf16, K);
     if (tune->vec > 0) p.sh.vec = tune->vec;
     if (tune->unroll > 0) p.sh.rw = tune->unroll;
     if (tune->bt > 0) p.sh.nrg = tune->bt;
@@ -217,6 +217,7 @@ hipError_t launch_fwd_lds(int K, const LdsPlan& p, const ConvPtrs& a, const LdsG
         case 5: return launch_fwd_lds_k5(p.sh, a, g, grid, s);
         case 7: return launch_fwd_lds_k7(p.sh, a, g, grid, s);
         case 9: return launch_fwd_lds_k9(p.sh, a, g, grid, s);
+        case 31: return launch_fwd_lds_k31(p.sh, a, g, grid, s);
     }
     return hipErrorInvalidConfiguration;
 }
@@ -228,20 +229,22 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
         case 5: return launch_bwd_lds_k5(p.sh, wdx, wdw, a, g, grid, s);
         case 7: return launch_bwd_lds_k7(p.sh, wdx, wdw, a, g, grid, s);
         case 9: return launch_bwd_lds_k9(p.sh, wdx, wdw, a, g, grid, s);
+        case 31: return launch_bwd_lds_k31(p.sh, wdx, wdw, a, g, grid, s);
     }
     return hipErrorInvalidConfiguration;
 }
 
 // algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged.
 // Measured on MI355X at T=131072, C=1024, K=7, bf16: both passes are fastest LDS-staged (the chip
-// sweeps one compact window of rows with every load of a tile issued at once); the sliding-window
-// kernels take what the LDS kernels are not built for (K > 9, narrow or unaligned rows).
+// sweeps one compact window of rows with every load of a tile issued at once). At K=31 (ALU-bound)
+// the LDS-staged forward still wins by ~17 % (C=1024 and 2048) but the fused backward does not fit
+// its registers, so it stays with the sliding-window kernel, like everything the LDS kernels are not
+// built for (K = 15, other sizes, narrow or unaligned rows).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
-    (void)bwd;
     const bool ok = lds_eligible(bf16, T, C, K, align_bits);
     if (tune && tune->algo == 2) return ok ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
-    return ok ? 2 : 1;
+    return (ok && (K <= 9 || !bwd)) ? 2 : 1;
 }
 
 // 256 threads x 4 x 16 B = one contiguous 16 KiB chunk per block
@@ -489,7 +492,7 @@ size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t 
     Plan p;
     if (make_plan(true, bf16, T, C, K, 0, nullptr, &p)) return 0;
     int slabs = p.nbt;
-    if (lds_eligible(bf16, T, C, K, 0)) {
+    if (choose_algo(true, nullptr, bf16, T, C, K, 0) == 2) {
         LdsPlan lp;
         if (make_lds_plan(true, bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
     }

@@ -97,6 +97,7 @@ NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
 NPLM_DECLARE_LDS_K(7)
 NPLM_DECLARE_LDS_K(9)
+NPLM_DECLARE_LDS_K(31)
 #undef NPLM_DECLARE_LDS_K
 NPLM_DECLARE_K(3)
 NPLM_DECLARE_K(5)
@@ -120,8 +121,8 @@ constexpr int default_unroll(bool bwd, int K, int vec) {
     if (K >= 15) return 8;
     return vec >= 8 ? 4 : 8;
 }
-// LDS-staged kernels are built for K <= 9.
-constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+// Kernel sizes the LDS-staged kernels are built for.
+constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 31; }
 // Default shapes (a block always owns 2 KiB of every row of its tile, 16-row tiles):
 //   forward : 4 wave-columns x 8 bytes per lane, 2 row groups of 8 rows, 4 loader waves; two x tiles
 //             of 16 + K-1 rows (88 KiB of LDS at K = 7).
@@ -129,7 +130,9 @@ constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K =
 //             (dy tile of 16 + K-1 rows, x tile of 16 rows) pairs = 152 KiB of the 160 KiB a CU has
 //             (exactly 160 KiB at K = 9). Four bytes per lane keep the 16-row register tile
 //             (dx accumulators + x rows + weights + dw/db) under the 128 registers 16 waves leave.
-constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16) {
+constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
+    if (K >= 15)   // long kernels: 1 KiB column blocks and 32-row tiles, so that tile + K-1 halo rows still fit twice
+        return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 2, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
     return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, 8, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
 }
 constexpr int default_maxt(bool bwd, int K, int vec) {
