@@ -133,7 +133,9 @@ constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K =
 constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
     if (K >= 15)   // long kernels: 1 KiB column blocks and 32-row tiles, so that tile + K-1 halo rows still fit twice
         return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 2, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
-    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, 8, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
+    // (K = 9 in bf16 needs more than 128 registers: 4 loader waves there, which leaves 168)
+    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, (bf16 && K >= 9) ? 4 : 8, 2}
+               : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
 }
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)bwd; (void)K; (void)vec;
