@@ -1,5 +1,5 @@
-// LDS-staged, software-pipelined kernels of the varlen depthwise conv (gfx950, wave64), for small
-// kernel sizes.
+// LDS-staged, software-pipelined kernels of the varlen depthwise conv (gfx950, wave64): both passes
+// for K <= 9, the forward also for K = 31.
 //
 // A block owns tiles of R = RW*NRG consecutive token rows x one column block of NCW*64*VEC channels
 // (2 KiB of every row at the default sizes). Its waves have two roles:

@@ -129,3 +129,44 @@ def test_registered_custom_ops_pass_opcheck_and_compile_without_graph_breaks():
     y64 = O.c_oracle_fwd(x.cpu(), cu_host, wl.weight, wl.bias)
     assert_act_close(y1, y64, torch.bfloat16, "compiled y")
     assert T < F
+
+
+def test_forward_and_backward_replay_correctly_from_a_hip_graph():
+    """The op allocates nothing, reads cu_seqlens on the device and never synchronises, so a training
+    step that contains it can be captured (reference: torch.compile + static shapes,
+    pure_pipeline.py:519-529). Replay several times with new contents in the static buffers, with eager
+    work and synchronisation between replays, and compare every replay with the eager result."""
+    torch.manual_seed(1)
+    lens = torch.tensor([100, 3, 512, 1, 408])
+    cu = torch.zeros(6, dtype=torch.int32)
+    cu[1:] = torch.cumsum(lens, 0)
+    cu = cu.to(DEV)
+    T, C, K = int(lens.sum()), 1024, 7
+    w = (torch.randn(C, K, device=DEV) * K ** -0.5).bfloat16()
+    b = (torch.randn(C, device=DEV) * 0.02).bfloat16()
+    sx = torch.zeros(T, C, device=DEV, dtype=torch.bfloat16)
+    sdy = torch.zeros_like(sx)
+    ws = torch.empty(npa.bwd_workspace_bytes(T, C, K, torch.bfloat16), dtype=torch.uint8, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up outside capture
+        npa.varlen_dwconv_fwd(sx, cu, w, b, residual=True)
+        npa.varlen_dwconv_bwd(sx, sdy, cu, w, residual=True, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gy = npa.varlen_dwconv_fwd(sx, cu, w, b, residual=True)
+        gdx, gdw, gdb = npa.varlen_dwconv_bwd(sx, sdy, cu, w, residual=True, workspace=ws)
+    for it in range(4):
+        x = torch.randn(T, C, device=DEV).bfloat16()
+        dy = torch.randn(T, C, device=DEV).bfloat16()
+        sx.copy_(x)
+        sdy.copy_(dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        ey = npa.varlen_dwconv_fwd(x, cu, w, b, residual=True)
+        edx, edw, edb = npa.varlen_dwconv_bwd(x, dy, cu, w, residual=True)
+        torch.cuda.synchronize()
+        assert torch.equal(gy, ey) and torch.equal(gdx, edx), f"replay {it}"
+        assert torch.equal(gdw, edw) and torch.equal(gdb, edb), f"replay {it}"
