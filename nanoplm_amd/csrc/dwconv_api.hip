@@ -162,7 +162,24 @@ bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     const int E = bf16 ? 2 : 4;
     if (!lds_kernel_size(K) || T < 1) return false;
     if (((long long)C * E) % 16 || align_bits % 16) return false;
-    return (long long)C * E >= 1024;   // narrower rows leave most of a block idle: sliding-window kernels
+    return (long long)C * E >= 1024;
+}
+
+// Whether they are also the faster choice. A block always owns a 2 KiB column block (1 KiB at K = 31)
+// of its rows and the grid's time follows the number of column blocks, so a row that fills its
+// column blocks poorly wastes lanes and loader slots. Measured on MI355X (T=131072, K=7, bf16 rows
+// of 1024 .. 6144 bytes and fp32 rows of 1024 .. 3072 bytes): LDS-staged wins for a single column
+// block filled to 5/8 or more and for several filled to 4/5 or more on average; the sliding-window
+// kernels win otherwise (e.g. rows of 1024, 2560 and 3072 bytes).
+bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    if (!lds_eligible(bf16, T, C, K, align_bits)) return false;
+    if (K > 9 && bwd) return false;        // K = 31: only the forward fits its registers
+    const LdsShapeSel sh = lds_default_shape(bwd, bf16, K);
+    const long long E = bf16 ? 2 : 4;
+    const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
+    const long long row_bytes = (long long)C * E;
+    const long long ncb = ceil_div(row_bytes, cb_bytes);
+    return ncb == 1 ? row_bytes * 8 >= cb_bytes * 5 : row_bytes * 5 >= ncb * cb_bytes * 4;
 }
 
 int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
@@ -241,10 +258,9 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
 // its registers, so it stays with the sliding-window kernel, like everything the LDS kernels are not
 // built for (K = 15, other sizes, narrow or unaligned rows).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
-    const bool ok = lds_eligible(bf16, T, C, K, align_bits);
-    if (tune && tune->algo == 2) return ok ? 2 : -NPLM_DWCONV_ETUNING;
+    if (tune && tune->algo == 2) return lds_eligible(bf16, T, C, K, align_bits) ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
-    return (ok && (K <= 9 || !bwd)) ? 2 : 1;
+    return lds_preferred(bwd, bf16, T, C, K, align_bits) ? 2 : 1;
 }
 
 // 256 threads x 4 x 16 B = one contiguous 16 KiB chunk per block
