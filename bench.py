@@ -116,7 +116,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", type=int, default=3, choices=[2, 3, 4, 5])
+    ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--residual", action="store_true",
                     help="fused residual variant: y = x + conv(x), dx = dy + conv^T(dy) (same traffic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
