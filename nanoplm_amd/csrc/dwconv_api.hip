@@ -86,7 +86,9 @@ int make_plan(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bi
     if (p.bw > wpb_max / p.bt) p.bw = wpb_max / p.bt;
     if (p.bw < 1 || (p.bw & (p.bw - 1))) return -NPLM_DWCONV_ETUNING;
     p.ncb = ceil_div(p.nwc, p.bw);
-    const int waves_per_cu = 8;
+    // waves the grid is sized for: 2 per SIMD keep the HBM-bound kernels streaming; the long kernels
+    // are ALU-bound and want every wave their registers allow (K=31 backward at C=2048: 848 -> 657 us)
+    const int waves_per_cu = K >= 15 ? 32 : 8;
     int nbt = tune->nbt > 0 ? tune->nbt : (kNumCU * waves_per_cu) / (p.ncb * p.bw * p.bt);
     const int nbt_useful = ceil_div(p.ntiles, p.bt);
     if (nbt > nbt_useful) nbt = nbt_useful;

@@ -3,10 +3,8 @@
 #ifdef NPLM_SWEEP
 // extra (dtype, VEC, U, launch-bounds) variants for the geometry sweeps
 #define NPLM_SWEEP_FWD                                                                     \
-    NPLM_FWD(true, 2, 16, 256) NPLM_FWD(true, 2, 8, 256) NPLM_FWD(true, 1, 16, 256)        \
-    NPLM_FWD(true, 4, 16, 256) NPLM_FWD(true, 4, 4, 256) NPLM_FWD(true, 2, 32, 256)
+    NPLM_FWD(true, 2, 16, 256) NPLM_FWD(true, 2, 4, 256)
 #define NPLM_SWEEP_BWD                                                                     \
-    NPLM_BWD(true, 1, 16, 256) NPLM_BWD(true, 1, 8, 256) NPLM_BWD(true, 2, 16, 256)        \
-    NPLM_BWD(true, 2, 4, 256) NPLM_BWD(true, 1, 32, 256) NPLM_BWD(true, 2, 8, 256)
+    NPLM_BWD(true, 1, 16, 256) NPLM_BWD(true, 1, 4, 256) NPLM_BWD(true, 1, 2, 256) NPLM_BWD(true, 2, 4, 256)
 #endif
 #include "dwconv_inst.inc"
