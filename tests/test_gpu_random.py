@@ -1,0 +1,77 @@
+"""Seeded random sweep over ragged length mixes, widths, kernel sizes, dtypes, kernel families and the
+residual flag, each case against the C oracle to the specification's tolerances. The length mixes
+lean on what breaks tiled kernels: zero-length entries, runs of sequences shorter than the kernel
+radius, boundaries on and around 8/16/32/64/256-row tile edges, one long sequence."""
+import random
+
+import pytest
+import torch
+
+import nanoplm_amd as npa
+from nanoplm_amd import _lib
+from nanoplm_amd.workloads import cu_from_lengths
+from oracle import dwconv_ref as O
+from tests.gpu_util import assert_act_close, assert_red_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _lengths(rng, total_hint):
+    kind = rng.choice(["tiny", "edges", "mixed", "one", "zeros"])
+    lens = []
+    if kind == "one":
+        return [rng.randint(1, total_hint)]
+    while sum(lens) < total_hint:
+        if kind == "tiny":
+            lens.append(rng.randint(1, 9))
+        elif kind == "edges":
+            lens.append(rng.choice([7, 8, 9, 15, 16, 17, 31, 32, 33, 63, 64, 65, 255, 256, 257]) + rng.choice([0, 0, 1]))
+        elif kind == "zeros":
+            lens.append(rng.choice([0, 0, 1, 2, 40, 200]))
+        else:
+            lens.append(rng.choice([rng.randint(1, 8), rng.randint(20, 512), rng.randint(400, 512)]))
+    return lens
+
+
+def _cases():
+    rng = random.Random(20260607)
+    out = []
+    for i in range(48):
+        K = rng.choice([1, 3, 5, 7, 7, 7, 9, 11, 15, 31])
+        dt = rng.choice([torch.bfloat16, torch.bfloat16, torch.float32])
+        wdt = rng.choice([dt, torch.float32])
+        C = rng.choice([8, 64, 100, 256, 512, 520, 768, 1024, 1024, 1536, 2048])
+        lens = _lengths(rng, rng.choice([60, 700, 3000, 9000]))
+        algo = rng.choice([0, 0, 1, 2])
+        out.append((i, K, dt, wdt, C, lens, algo, rng.random() < 0.4, rng.random() < 0.8))
+    return out
+
+
+@pytest.mark.parametrize("case", _cases(), ids=lambda c: f"{c[0]}-K{c[1]}-C{c[4]}-{'bf16' if c[2] == torch.bfloat16 else 'f32'}-a{c[6]}")
+def test_random_case_matches_oracle(case):
+    i, K, dt, wdt, C, lens, algo, residual, with_bias = case
+    print(f"[case] #{i} K={K} C={C} {dt}/{wdt} algo={algo} residual={residual} S={len(lens)} T={sum(lens)}", flush=True)
+    g = torch.Generator().manual_seed(1000 + i)
+    T = sum(lens)
+    x = torch.randn(T, C, generator=g).to(dt)
+    dy = torch.randn(T, C, generator=g).to(dt)
+    w = (torch.randn(C, K, generator=g) * K ** -0.5).to(wdt)
+    b = (torch.randn(C, generator=g) * 0.02).to(wdt) if with_bias else None
+    cu = cu_from_lengths(torch.tensor(lens))
+    tune = _lib.Tuning(algo=algo) if algo else None
+    xd, dyd, wd, cud = x.to(DEV), dy.to(DEV), w.to(DEV), cu.to(DEV)
+    bd = None if b is None else b.to(DEV)
+    try:
+        y = npa.varlen_dwconv_fwd(xd, cud, wd, bd, residual=residual, tuning=tune)
+        dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, residual=residual, tuning=tune)
+    except RuntimeError as e:
+        if algo == 2 and "not available" in str(e):
+            pytest.skip("LDS-staged kernels are not built for this shape")   # narrow rows, other K
+        raise
+    y64 = O.c_oracle_fwd(x, cu, w, b, residual=residual)
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w, residual=residual)
+    assert_act_close(y, y64, dt, "y")
+    assert_act_close(dx, dx64, dt, "dx")
+    assert_red_close(dw, dw64, "dw")
+    assert_red_close(db, db64, "db")
