@@ -186,4 +186,22 @@ struct SeqCursor {
     }
 };
 
+// Which of the K taps of output row t stay inside the cursor's interval: bit m is set iff row
+// t - P + m lies in [cs, ce). One scalar word (K <= 32) per row instead of two compares per tap;
+// the kernels test its bits with scalar instructions and select, never multiply by zero.
+template <int K>
+__device__ __forceinline__ uint32_t row_tap_mask(const SeqCursor& sc, int t) {
+    static_assert(K <= 32, "one mask bit per tap");
+    constexpr int P = (K - 1) / 2;
+    int lo = sc.cs - (t - P), hi = sc.ce - (t - P);     // valid taps: lo <= m < hi
+    lo = lo < 0 ? 0 : lo;
+    hi = hi > K ? K : hi;
+    const uint32_t m = hi > lo ? (uint32_t)(((1ull << hi) - 1ull) & ~((1ull << lo) - 1ull)) : 0u;
+#if defined(__HIP_DEVICE_COMPILE__)
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)m);
+#else
+    return m;
+#endif
+}
+
 }  // namespace nplm

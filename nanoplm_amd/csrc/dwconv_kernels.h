@@ -216,10 +216,10 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
                                 float acc[VEC];
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) acc[v] = bias[v];
+                                const uint32_t taps = row_tap_mask<K>(sc, t);
 #pragma unroll
                                 for (int k = 0; k < K; ++k) {
-                                    const int j = t + k - P;
-                                    const bool ok = (j >= sc.cs) && (j < sc.ce);
+                                    const bool ok = (taps >> k) & 1u;      // row t + k - P is in t's sequence
 #pragma unroll
                                     for (int v = 0; v < VEC; ++v) {
                                         const float xv = ok ? win[RG::slot(ph, u + k)][v] : 0.f;
@@ -383,10 +383,10 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                         acc[v] = 0.f;
                                         if constexpr (WDW) dba[v] += gw[RG::slot(ph, u + P)][v];
                                     }
+                                    const uint32_t taps = row_tap_mask<K>(sc, t);
 #pragma unroll
                                     for (int m = 0; m < K; ++m) {
-                                        const int j = t + m - P;
-                                        const bool ok = (j >= sc.cs) && (j < sc.ce);
+                                        const bool ok = (taps >> m) & 1u;  // row t + m - P is in t's sequence
 #pragma unroll
                                         for (int v = 0; v < VEC; ++v) {
                                             const float gv = ok ? gw[RG::slot(ph, u + m)][v] : 0.f;

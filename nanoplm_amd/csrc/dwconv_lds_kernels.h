@@ -194,17 +194,13 @@ __device__ __forceinline__ void pin_regs(float (&r)[N]) {
 template <int RW, int K>
 __device__ __forceinline__ void wave_tap_masks(SeqCursor sc, const int32_t* __restrict__ cu, int S, int T, int tf,
                                                uint32_t (&vm)[RW]) {
-    constexpr int P = (K - 1) / 2;
 #pragma unroll
     for (int u = 0; u < RW; ++u) {
         const int t = tf + u;
         uint32_t m = 0;
         if (t < T) {
             sc.advance(cu, S, T, t);
-            int lo = sc.cs - (t - P), hi = sc.ce - (t - P);     // valid taps: lo <= m < hi
-            lo = lo < 0 ? 0 : lo;
-            hi = hi > K ? K : hi;
-            if (hi > lo) m = (uint32_t)(((1ull << hi) - 1ull) & ~((1ull << lo) - 1ull));
+            m = row_tap_mask<K>(sc, t);
         }
         vm[u] = m;
     }
