@@ -148,13 +148,7 @@ __device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
     r.to_f32(f);
 }
 
-// Per-output-row tap limits of a wave's RW rows: tap row g is valid for output u iff lo[u] <= g < hi[u].
-template <int RW>
-struct WaveBounds {
-    int lo[RW], hi[RW];
-};
-
-// The expensive half of the boundary lookup: position the cursor on the sequence of row tf (a chain
+// The expensive part of the boundary lookup: position the cursor on the sequence of row tf (a chain
 // of dependent scalar loads). The compute waves run it for the NEXT tile right before the tile
 // barrier, where they would otherwise idle until the loaders' data has landed.
 // Returns true when every tap of rows tf .. tf+RW-1 lies inside that one sequence.
@@ -164,20 +158,6 @@ __device__ __forceinline__ bool wave_locate(SeqCursor& sc, const int32_t* __rest
     sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
     const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
     return (tf - P >= sc.cs) && (tl + P < sc.ce);
-}
-
-// The cheap half, only needed for a wave whose rows touch a sequence boundary: walk the cursor over
-// the RW rows. `sc` is taken by value so the caller's cursor keeps pointing at row tf.
-template <int RW>
-__device__ __forceinline__ void wave_row_bounds(SeqCursor sc, const int32_t* __restrict__ cu, int S, int T, int tf,
-                                                WaveBounds<RW>& wb) {
-#pragma unroll
-    for (int u = 0; u < RW; ++u) {
-        const int t = tf + u;
-        if (t < T) sc.advance(cu, S, T, t);
-        wb.lo[u] = sc.cs;
-        wb.hi[u] = sc.ce;
-    }
 }
 
 // Empty volatile asm that takes N registers in and out: orders the instructions that produce them
@@ -312,17 +292,16 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         }
                     }
                 } else {
-                    WaveBounds<RW> wb;
-                    wave_row_bounds<RW>(sc, cu, S, T, tf, wb);
+                    uint32_t vm[RW];
+                    wave_tap_masks<RW, K>(sc, cu, S, T, tf, vm);
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
                         lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
-                        const int gr = tf - P + j;
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
-                                const bool ok = (gr >= wb.lo[u]) && (gr < wb.hi[u]);
+                                const bool ok = (vm[u] >> (j - u)) & 1u;
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) {
                                     const float xv = ok ? xr[v] : 0.f;
