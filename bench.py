@@ -65,6 +65,12 @@ class HipEvents:
                 raise RuntimeError(f"hipEventCreate failed: {rc}")
             self.ev.append(e)
 
+    @staticmethod
+    def record_raw(event, stream):
+        rc = _hip().hipEventRecord(ctypes.c_void_p(event), ctypes.c_void_p(stream))
+        if rc:
+            raise RuntimeError(f"hipEventRecord failed: {rc}")
+
     def record(self, i, stream):
         rc = self.hip.hipEventRecord(self.ev[i], ctypes.c_void_p(stream))
         if rc:
@@ -119,6 +125,9 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=[1, 2, 3, 4, 5])
     ap.add_argument("--residual", action="store_true",
                     help="fused residual variant: y = x + conv(x), dx = dy + conv^T(dy) (same traffic)")
+    ap.add_argument("--gated", action="store_true",
+                    help="gated variant: input z = [x_proj | gate] of width 2C, conv over x_proj * silu(gate) "
+                         "(informational; per-kernel figures then bracket backward + finalize together)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=65536)
     args = ap.parse_args()
@@ -142,20 +151,30 @@ def main():
     T, C, K, S = wl.T, wl.C, wl.K, wl.S
     fwd_bwd = wl.passes == "fwd+bwd"
     NSET = 3
+    if args.gated and not fwd_bwd:
+        sys.exit("--gated needs a forward+backward configuration (3, 4 or 5)")
     xs = [d.x] + [torch.randn(T, C, device=dev).to(wl.dtype) for _ in range(NSET - 1)]
+    if args.gated:       # z = [x_proj | gate]; dz has the same shape
+        xs = [torch.randn(T, 2 * C, device=dev).to(wl.dtype) for _ in range(NSET)]
     gs = [d.dy] + [torch.randn(T, C, device=dev).to(wl.dtype) for _ in range(NSET - 1)]
     ys = [torch.empty_like(d.x) for _ in range(NSET)]
-    dxs = [torch.empty_like(d.x) for _ in range(NSET)]
+    dxs = [torch.empty_like(xs[0]) for _ in range(NSET)]
     dw = torch.empty((C, K), dtype=torch.float32, device=dev)
     db = torch.empty((C,), dtype=torch.float32, device=dev)
     act = _lib.BF16 if wl.dtype == torch.bfloat16 else _lib.F32
-    ws_bytes = int(lib.nplm_dwconv_bwd_workspace_bytes(T, C, K, act))
+    ws_bytes = int((lib.nplm_dwconv_gated_bwd_workspace_bytes if args.gated else lib.nplm_dwconv_bwd_workspace_bytes)(T, C, K, act))
+    if args.gated and ws_bytes == 0:
+        sys.exit("the fused gated kernels are not built for this configuration")
     ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     cu, w, b = d.cu_seqlens, d.weight, d.bias
     flags = _lib.RESIDUAL if args.residual else 0
     def fwd(i):
         j = i % NSET
+        if args.gated:
+            _lib.check(lib.nplm_dwconv_gated_fwd(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(),
+                                                 ys[j].data_ptr(), T, C, K, S, act, act, flags, stream), "nplm_dwconv_gated_fwd")
+            return
         _lib.check(lib.nplm_dwconv_fwd_ex(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(),
                                           ys[j].data_ptr(), T, C, K, S, act, act, flags, stream), "nplm_dwconv_fwd_ex")
 
@@ -163,7 +182,12 @@ def main():
         j = i % NSET
         args_ = (xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(),
                  db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act)
-        rc = lib.nplm_dwconv_bwd_ex(*args_, flags, stream) if t is None else lib.nplm_dwconv_bwd_tuned(*args_, stream, t)
+        if args.gated:
+            rc = lib.nplm_dwconv_gated_bwd(*args_, flags, stream)
+            if t is not None and t.mid_event:      # no mid-call event on this entry point: mark the end instead
+                HipEvents.record_raw(t.mid_event, stream)
+        else:
+            rc = lib.nplm_dwconv_bwd_ex(*args_, flags, stream) if t is None else lib.nplm_dwconv_bwd_tuned(*args_, stream, t)
         _lib.check(rc, "nplm_dwconv_bwd")
 
     def step(i):
@@ -225,28 +249,35 @@ def main():
     ev = evs[0]
     fwd_avg = statistics.fmean(fwd_us)
     fwd_bytes = wl.algorithmic_bytes("fwd")
+    bwd_bytes = wl.algorithmic_bytes("bwd") if fwd_bwd else 0
+    if args.gated:       # z is read once more per pass and dz is twice as wide as dx
+        tce = T * C * d.x.element_size()
+        fwd_bytes += tce
+        bwd_bytes += 2 * tce
+    step_bytes = fwd_bytes + bwd_bytes
 
     def roof(nbytes, us, kernel):
         gbps = nbytes / us / 1e3
         return {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                "traffic": MEASURED_TRAFFIC.get((wl.name, kernel)), "kernel": kernel, "avg_us": us,
+                "traffic": None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel)), "kernel": kernel, "avg_us": us,
                 "algorithmic_bytes": nbytes}
 
     out = {
         "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
-                  if args.config == 3 else f"varlen dwconv {wl.passes} tokens/s ({wl.name})",
+                  if args.config == 3 and not args.gated else
+                  f"varlen {'gated ' if args.gated else ''}dwconv {wl.passes} tokens/s ({wl.name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
         "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
-                   "rotating_sets": NSET, "residual": bool(args.residual)},
-        "step_algorithmic_bytes": wl.algorithmic_bytes(),
-        "step_GBps": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9,
-        "step_frac_of_hbm_peak": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                   "rotating_sets": NSET, "residual": bool(args.residual), "gated": bool(args.gated)},
+        "step_algorithmic_bytes": step_bytes,
+        "step_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
+        "step_frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
     }
     if fwd_bwd:
-        out["roofline"] = roof(wl.algorithmic_bytes("bwd"), statistics.fmean(bwd_us), "backward")
+        out["roofline"] = roof(bwd_bytes, statistics.fmean(bwd_us), "backward")
         out["roofline_fwd"] = roof(fwd_bytes, fwd_avg, "forward")
         out["finalize_avg_us"] = statistics.fmean(fin_us)
     else:

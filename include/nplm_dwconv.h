@@ -63,6 +63,7 @@ extern "C" {
 #define NPLM_DWCONV_EWORKSPACE 6  /* workspace NULL, misaligned (256 B) or smaller than required */
 #define NPLM_DWCONV_ECU        7  /* check_cu: cu[0] != 0, cu decreasing, or cu[S] != T */
 #define NPLM_DWCONV_EFLAGS     9  /* unknown bits set in `flags` (8 is used by the internal tuning interface) */
+#define NPLM_DWCONV_EUNSUPPORTED 10 /* gated entry points: shape outside what the fused kernels are built for */
 
 /* flags of the _ex entry points */
 #define NPLM_DWCONV_RESIDUAL 1u   /* fuse the residual connection: y = x + conv(x), dx = dy + conv^T(dy) */
@@ -126,6 +127,29 @@ int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const v
                        void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,
                        int64_t T, int32_t C, int32_t K, int32_t S,
                        int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
+
+/*
+ * Gated variants: the conv over h = x_proj * silu(gate) with the gate product fused into the conv's
+ * loads, for a conv placed inside the SwiGLU MLP (ModernBertSwiGLUMLP.forward, modeling.py:300-302:
+ * `x_proj, gate = self.Wi(x).chunk(2, dim=-1)`, then `F.silu(gate) * x_proj`).
+ *   z, dz : [T, 2C] row-major, act_dtype; columns [0, C) are x_proj, columns [C, 2C) are gate
+ *   y, dy : [T, C]
+ *   y  = conv(h; w, b), h = z[:, :C] * silu(z[:, C:])           (h is formed in fp32, never stored)
+ *   dz = [dh * silu(gate) | dh * x_proj * silu'(gate)], dh = conv^T(dy; w); dw, db as for conv(h)
+ * This saves writing h and reading it back (forward) and the separate elementwise backward (backward).
+ * Built for K in {3,5,7,9}, C * elemsize a multiple of 16 bytes and at least 1 KiB, 16-byte aligned
+ * z / y / dy / dz; anything else returns -NPLM_DWCONV_EUNSUPPORTED and launches nothing (callers then
+ * compose the unfused ops). `flags` as for nplm_dwconv_fwd_ex (the residual applies to h).
+ * nplm_dwconv_gated_bwd_workspace_bytes returns 0 for unsupported shapes.
+ */
+int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const void* b, void* y,
+                          int64_t T, int32_t C, int32_t K, int32_t S,
+                          int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
+size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype);
+int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, const void* w,
+                          void* dz, float* dw, float* db, void* workspace, size_t workspace_bytes,
+                          int64_t T, int32_t C, int32_t K, int32_t S,
+                          int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
  * Debug helper: copies cu to the host (synchronises `stream`) and verifies the preconditions.

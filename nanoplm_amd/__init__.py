@@ -18,6 +18,13 @@ from .padded import (  # noqa: F401
     right_padded_cu_seqlens,
     unpad_input,
 )
+from .gated import (  # noqa: F401
+    GatedVarlenDWConv1dFunction,
+    gated_dwconv_bwd,
+    gated_dwconv_fwd,
+    gated_supported,
+    gated_varlen_dwconv,
+)
 from .hygiene import conv_parameters, split_conv_parameters  # noqa: F401
 
 __version__ = "0.1.0"

@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libnplm_dwconv.so")
 F32 = 0
 BF16 = 1
 RESIDUAL = 1    # NPLM_DWCONV_RESIDUAL
+EUNSUPPORTED = 10   # NPLM_DWCONV_EUNSUPPORTED
 
 # every symbol include/nplm_dwconv.h declares
 PUBLIC_SYMBOLS = (
@@ -24,6 +25,9 @@ PUBLIC_SYMBOLS = (
     "nplm_dwconv_bwd_workspace_bytes",
     "nplm_dwconv_bwd",
     "nplm_dwconv_bwd_ex",
+    "nplm_dwconv_gated_fwd",
+    "nplm_dwconv_gated_bwd_workspace_bytes",
+    "nplm_dwconv_gated_bwd",
     "nplm_dwconv_check_cu",
 )
 
@@ -67,6 +71,12 @@ def load():
     lib.nplm_dwconv_bwd.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_ex.argtypes = bwd_args[:-1] + [ctypes.c_uint32, vp]
     lib.nplm_dwconv_bwd_ex.restype = ctypes.c_int
+    lib.nplm_dwconv_gated_fwd.argtypes = fwd_args[:-1] + [ctypes.c_uint32, vp]
+    lib.nplm_dwconv_gated_fwd.restype = ctypes.c_int
+    lib.nplm_dwconv_gated_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
+    lib.nplm_dwconv_gated_bwd_workspace_bytes.restype = sz
+    lib.nplm_dwconv_gated_bwd.argtypes = bwd_args[:-1] + [ctypes.c_uint32, vp]
+    lib.nplm_dwconv_gated_bwd.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_tuned.argtypes = bwd_args + [ctypes.POINTER(Tuning)]
     lib.nplm_dwconv_bwd_tuned.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_slabs.argtypes = [i64, i32, i32, i32, ctypes.POINTER(Tuning)]

@@ -184,12 +184,13 @@ bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t ali
     return ncb == 1 ? row_bytes * 8 >= cb_bytes * 5 : row_bytes * 5 >= ncb * cb_bytes * 4;
 }
 
-int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
+int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out,
+                  bool gated = false) {
     LdsPlan p{};
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    p.sh = lds_default_shape(bwd, bf16, K);
+    p.sh = gated ? lds_gated_shape(bwd, bf16) : lds_default_shape(bwd, bf16, K);
     if (tune->vec > 0) p.sh.vec = tune->vec;
     if (tune->unroll > 0) p.sh.rw = tune->unroll;
     if (tune->bt > 0) p.sh.nrg = tune->bt;
@@ -199,9 +200,11 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     const long long cb_bytes = (long long)p.sh.ncw * 64 * p.sh.vec * E;
     const long long row_bytes = (long long)C * E;
     p.R = p.sh.rw * p.sh.nrg;
-    const size_t shmem = (size_t)p.sh.nbuf * ((size_t)(p.R + K - 1) + (bwd ? p.R : 0)) * cb_bytes;
+    const size_t tile_rows = gated ? (bwd ? (size_t)(p.R + K - 1) + 2 * (size_t)p.R : 2 * (size_t)(p.R + K - 1))
+                                   : (size_t)(p.R + K - 1) + (bwd ? p.R : 0);
+    const size_t shmem = (size_t)p.sh.nbuf * tile_rows * cb_bytes;
     if (shmem > kLdsBytesPerCU || cb_bytes % 1024) return -NPLM_DWCONV_ETUNING;
-    if ((long long)(p.R + K) * row_bytes + row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
+    if ((long long)(p.R + K) * row_bytes * (gated ? 2 : 1) + 2 * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
     p.ncb = ceil_div(row_bytes, cb_bytes);
     p.ntiles = ceil_div(T, p.R);
     int nbt = tune->nbt > 0 ? tune->nbt : kNumCU / p.ncb;
@@ -288,6 +291,14 @@ hipError_t fill_zero(float* p, long long n, hipStream_t s) {
 }
 
 // launch flags of the kernels (W_BF16 | W_RESIDUAL) from the ABI's weight dtype and flags
+// Shapes the gated (z = [u | g]) kernels are built for.
+bool gated_supported(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    const int E = bf16 ? 2 : 4;
+    if (!lds_gated_kernel_size(K) || T < 1) return false;
+    if (((long long)C * E) % 16 || align_bits % 16) return false;
+    return (long long)C * E >= 1024;
+}
+
 int kernel_w_flags(int32_t w_dtype, uint32_t flags) {
     return (w_dtype == NPLM_DWCONV_BF16 ? W_BF16 : 0) | ((flags & NPLM_DWCONV_RESIDUAL) ? W_RESIDUAL : 0);
 }
@@ -469,6 +480,86 @@ extern "C" {
 
 int nplm_dwconv_version(void) { return kVersion; }
 
+int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const void* b, void* y, int64_t T,
+                          int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags,
+                          void* stream) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    if (T == 0) return 0;
+    if (!z || !cu || !w || !y) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
+    if (!gated_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)y)) return -NPLM_DWCONV_EUNSUPPORTED;
+    LdsPlan lp;
+    rc = make_lds_plan(false, bf16, T, C, K, nullptr, &lp, true);
+    if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
+    const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
+    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+    const dim3 grid(lp.ncb * lp.nbt);
+    hipStream_t s = (hipStream_t)stream;
+    switch (K) {
+        case 3: return (int)launch_fwd_lds_gated_k3(bf16, la, g, grid, s);
+        case 5: return (int)launch_fwd_lds_gated_k5(bf16, la, g, grid, s);
+        case 7: return (int)launch_fwd_lds_gated_k7(bf16, la, g, grid, s);
+        case 9: return (int)launch_fwd_lds_gated_k9(bf16, la, g, grid, s);
+    }
+    return -NPLM_DWCONV_EUNSUPPORTED;
+}
+
+size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
+    if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    if (!gated_supported(bf16, T, C, K, 0)) return 0;
+    LdsPlan lp;
+    if (make_lds_plan(true, bf16, T, C, K, nullptr, &lp, true)) return 0;
+    const size_t bytes = (size_t)lp.nbt * (K + 1) * C * sizeof(float);
+    return (bytes + 255) & ~(size_t)255;
+}
+
+int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, const void* w, void* dz, float* dw,
+                          float* db, void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K,
+                          int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dw || !db) return -NPLM_DWCONV_ENULL;
+    if (T == 0) {
+        hipError_t e = fill_zero(dw, (long long)C * K, s);
+        if (e == hipSuccess) e = fill_zero(db, C, s);
+        return (int)e;
+    }
+    if (!z || !dy || !cu || !w || !dz) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
+    if (!gated_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
+    LdsPlan lp;
+    rc = make_lds_plan(true, bf16, T, C, K, nullptr, &lp, true);
+    if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
+    const size_t slab_bytes = (size_t)(K + 1) * C * sizeof(float);
+    if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab_bytes * (size_t)lp.nbt)
+        return -NPLM_DWCONV_EWORKSPACE;
+    float* part = reinterpret_cast<float*>(workspace);
+    const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
+    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+    const dim3 grid(lp.ncb * lp.nbt);
+    hipError_t e = hipErrorInvalidConfiguration;
+    switch (K) {
+        case 3: e = launch_bwd_lds_gated_k3(bf16, la, g, grid, s); break;
+        case 5: e = launch_bwd_lds_gated_k5(bf16, la, g, grid, s); break;
+        case 7: e = launch_bwd_lds_gated_k7(bf16, la, g, grid, s); break;
+        case 9: e = launch_bwd_lds_gated_k9(bf16, la, g, grid, s); break;
+    }
+    if (e != hipSuccess) return (int)e;
+    const long long n_out = (long long)(K + 1) * C;
+    hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                       (const float*)part, lp.nbt, C, K, dw, db);
+    return (int)hipGetLastError();
+}
+
 const char* nplm_dwconv_strerror(int code) {
     if (code == 0) return "success";
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -481,6 +572,7 @@ const char* nplm_dwconv_strerror(int code) {
         case NPLM_DWCONV_EWORKSPACE: return "nplm_dwconv: workspace NULL, not 256-byte aligned, or too small";
         case NPLM_DWCONV_ECU: return "nplm_dwconv: cu_seqlens must start at 0, be non-decreasing and end at T";
         case NPLM_DWCONV_EFLAGS: return "nplm_dwconv: unknown bits set in flags";
+        case NPLM_DWCONV_EUNSUPPORTED: return "nplm_dwconv: shape not supported by the fused gated kernels";
         case NPLM_DWCONV_ETUNING: return "nplm_dwconv: geometry override not available in this build";
     }
     return "nplm_dwconv: unknown error code";

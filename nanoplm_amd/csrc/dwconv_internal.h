@@ -93,6 +93,14 @@ struct LdsShapeSel {
                                     hipStream_t s);                                                       \
     hipError_t launch_bwd_lds_k##KK(const LdsShapeSel& sh, bool wdx, bool wdw, const ConvPtrs& p,         \
                                     const LdsGeo& g, dim3 grid, hipStream_t s);
+#define NPLM_DECLARE_LDS_GATED_K(KK)                                                                      \
+    hipError_t launch_fwd_lds_gated_k##KK(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s); \
+    hipError_t launch_bwd_lds_gated_k##KK(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+NPLM_DECLARE_LDS_GATED_K(3)
+NPLM_DECLARE_LDS_GATED_K(5)
+NPLM_DECLARE_LDS_GATED_K(7)
+NPLM_DECLARE_LDS_GATED_K(9)
+#undef NPLM_DECLARE_LDS_GATED_K
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
 NPLM_DECLARE_LDS_K(7)
@@ -137,6 +145,15 @@ constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
     return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, (bf16 && K >= 9) ? 4 : 8, 2}
                : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
 }
+// Gated kernels (z = [u | g] input): 1 KiB column blocks, so that a u tile and a g tile fit where the plain
+// kernels hold one x tile: 4 wave-columns x 4 bytes per lane, 2 row groups, 4 loader waves. The gate
+// costs two transcendentals per element read, so the forward takes 32-row tiles (16 rows per wave: the
+// K-1 halo rows it re-gates weigh less; 2 x 2 x 38 KiB = 152 KiB of LDS at K = 7), the backward 16-row
+// tiles (2 x (22 + 16 + 16) KiB = 108 KiB).
+constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16) {
+    return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, 2, 4, 4, 2};
+}
+constexpr bool lds_gated_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)bwd; (void)K; (void)vec;
     return 256;

@@ -148,6 +148,23 @@ __device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
     r.to_f32(f);
 }
 
+// SwiGLU gate of the reference MLP (modeling.py:300-302: F.silu(gate) * x_proj), in fp32:
+// sig = 1 / (1 + 2^(-g log2 e)); h = u * g * sig. Also what the backward needs of it.
+__device__ __forceinline__ float sigmoid_f32(float g) {
+    return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g));
+}
+__device__ __forceinline__ float gate_mul(float u, float g) { return u * g * sigmoid_f32(g); }
+
+// One lane's slice of a gated input row out of LDS: h[v] = u[v] * silu(g[v]).
+template <bool BF16, int VEC>
+__device__ __forceinline__ void lds_read_gated_row(const char* pu, const char* pg, float (&h)[VEC]) {
+    float u[VEC], g[VEC];
+    lds_read_row<BF16, VEC>(pu, u);
+    lds_read_row<BF16, VEC>(pg, g);
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) h[v] = gate_mul(u[v], g[v]);
+}
+
 // The expensive part of the boundary lookup: position the cursor on the sequence of row tf (a chain
 // of dependent scalar loads). The compute waves run it for the NEXT tile right before the tile
 // barrier, where they would otherwise idle until the loaders' data has landed.
@@ -191,16 +208,22 @@ __device__ __forceinline__ void wave_tap_masks(SeqCursor sc, const int32_t* __re
 // =============================================================================================
 // NBUF = 2: one tile in flight while one is consumed. NBUF = 3: two tiles in flight (the loaders wait
 // only for the older one), which keeps HBM busy when a single tile's latency exceeds its compute time.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, int NBUF>
+//
+// GATED: x is z = [u | g] of shape [T, 2C] (the SwiGLU MLP's Wi output, modeling.py:300-302) and the
+// conv runs over h = u * silu(g), formed in registers as rows are read out of LDS; a buffer then
+// holds a u tile followed by a g tile, and y is still [T, C].
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, int NBUF, bool GATED = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
                       const void* __restrict__ b, void* __restrict__ y, const LdsGeo g) {
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     using Row = RowVec<BF16, VEC>;
-    constexpr int CNT = (SH::NROWS * SH::NPIECE + NWL - 1) / NWL;     // loads per loader wave per tile
+    constexpr int CNT = (SH::NROWS * SH::NPIECE + NWL - 1) / NWL;     // loads per loader wave per tile and tensor
+    constexpr int BUF_BYTES = SH::TILE_BYTES * (GATED ? 2 : 1);
     static_assert(NBUF == 2 || NBUF == 3, "two or three tile buffers");
-    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x TILE_BYTES
+    static_assert(!GATED || NBUF == 2, "the gated forward is double-buffered");
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x BUF_BYTES
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
@@ -213,6 +236,14 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     const int col_byte0 = cb * SH::CB_BYTES;
     const int valid_bytes = (rowb - col_byte0 < SH::CB_BYTES) ? rowb - col_byte0 : SH::CB_BYTES;
     const int ntl = (g.ntiles - tb + g.nbt - 1) / g.nbt;   // tiles of this block (>= 1), same for all waves
+    const size_t in_row_bytes = GATED ? 2 * row_bytes : row_bytes;   // pitch of x (z when gated)
+    auto stage_tile = [&](char* buf, int first_row) {
+        stage_rows_fixed<SH, CNT>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
+                                  NWL, lane);
+        if constexpr (GATED)
+            stage_rows_fixed<SH, CNT>(x, buf + SH::TILE_BYTES, first_row, SH::NROWS, T, in_row_bytes, rowb + col_byte0,
+                                      valid_bytes, wv - SH::NWC, NWL, lane);
+    };
 
     // compute-wave coordinates (meaningless but harmless for loader waves)
     const int wc = wv % NCW;
@@ -229,11 +260,9 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
     if (is_loader) {
-        stage_rows_fixed<SH, CNT>(x, lds_raw, tb * R - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
-                                  NWL, lane);
+        stage_tile(lds_raw, tb * R - P);
         if (NBUF == 3 && ntl > 1) {
-            stage_rows_fixed<SH, CNT>(x, lds_raw + SH::TILE_BYTES, (tb + g.nbt) * R - P, SH::NROWS, T, row_bytes,
-                                      col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
+            stage_tile(lds_raw + BUF_BYTES, (tb + g.nbt) * R - P);
             wait_vmem_but<CNT>();     // tile 0 has landed, tile 1 may still be in flight
         } else {
             wait_vmem_all();
@@ -256,15 +285,14 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     int bcur = 0;                       // buffer of tile `it`
     for (int it = 0; it < ntl; ++it) {
         const int t0 = (tb + it * g.nbt) * R;
-        char* cur = lds_raw + bcur * SH::TILE_BYTES;
+        char* cur = lds_raw + bcur * BUF_BYTES;
         if (is_loader) {
             // stage tile it + NBUF - 1 into the buffer freed by the barrier that ended iteration it - 1,
             // then wait until tile it + 1 has landed
             const int ahead = NBUF - 1;
             if (it + ahead < ntl) {
                 const int bnew = (bcur + ahead) % NBUF;
-                stage_rows_fixed<SH, CNT>(x, lds_raw + bnew * SH::TILE_BYTES, t0 + ahead * g.nbt * R - P, SH::NROWS, T,
-                                          row_bytes, col_byte0, valid_bytes, wv - SH::NWC, NWL, lane);
+                stage_tile(lds_raw + bnew * BUF_BYTES, t0 + ahead * g.nbt * R - P);
                 if (NBUF == 3) wait_vmem_but<CNT>(); else wait_vmem_all();
             } else {
                 wait_vmem_all();
@@ -282,7 +310,8 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
-                        lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+                        if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
+                        else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
@@ -297,7 +326,8 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
-                        lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+                        if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
+                        else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
@@ -336,14 +366,20 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 //     dx[t] = sum_m w[K-1-m] * dy[t-P+m],   dw[K-1-m] += x[t] * dy[t-P+m],   db += dy[t].
 // So only the dy tile carries halo rows; the x tile is exactly the R rows of the tile.
 // LDS: [2 buffers][dy tile (R+K-1 rows), x tile (R rows, only when dw/db are wanted)].
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW>
+//
+// GATED: x is z = [u | g] of shape [T, 2C], the conv ran over h = u * silu(g), and dx is dz [T, 2C]:
+// a buffer holds the dy tile, a u tile and a g tile; h rows (for dw) and the two halves of dz
+//     du = dh * silu(g),   dg = dh * u * sig(g) * (1 + g * (1 - sig(g))),   dh = the conv's dx
+// are formed in registers from the staged u and g rows.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                       const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     constexpr int XT_BYTES = R * SH::CB_BYTES;
-    constexpr int BUF_BYTES = SH::TILE_BYTES + (WDW ? XT_BYTES : 0);
+    constexpr int BUF_BYTES = SH::TILE_BYTES + (WDW ? XT_BYTES : 0) * (GATED ? 2 : 1);
+    static_assert(!GATED || (WDX && WDW), "the gated backward always produces dz, dw and db");
     using Row = RowVec<BF16, VEC>;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
 
@@ -369,14 +405,21 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     const int out_voff = c0 * E;
     const int lw = wv - SH::NWC;
 
+    const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;    // pitch of x and dx (z and dz when gated)
+    auto stage_x = [&](char* buf, int t0, int l, int nl) {
+        stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, x_row_bytes, col_byte0, valid_bytes, l, nl, lane);
+        if constexpr (GATED)
+            stage_rows<SH>(x, buf + SH::TILE_BYTES + XT_BYTES, t0, R, T, x_row_bytes, rowb + col_byte0, valid_bytes, l, nl,
+                           lane);
+    };
     auto stage_both = [&](char* buf, int t0) {
-        // with two or more loader waves, even ones take the dy tile and odd ones the x tile
+        // with two or more loader waves, even ones take the dy tile and odd ones the x tile(s)
         if constexpr (WDW && NWL >= 2) {
-            if (lw & 1) stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, row_bytes, col_byte0, valid_bytes, lw >> 1, NWL / 2, lane);
+            if (lw & 1) stage_x(buf, t0, lw >> 1, NWL / 2);
             else        stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane);
         } else {
             stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
-            if constexpr (WDW) stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+            if constexpr (WDW) stage_x(buf, t0, lw, NWL);
         }
     };
 
@@ -415,13 +458,67 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
                 const char* lpx = cur + SH::TILE_BYTES + loff;     // x : staged row u <-> global row tf + u
-                const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
+                const rsrc_t ro = rows_rsrc(dx, tf, T, x_row_bytes);
+                // Gated: per element of the wave's x rows, the two factors everything else needs:
+                //   gs = silu(g) / ... = g * sig(g)              (h = u * gs, du = dh * gs)
+                //   gd = u * sig(g) * (1 + g * (1 - sig(g)))     (dg = dh * gd)
+                float gs[GATED ? RW : 1][VEC], gd[GATED ? RW : 1][VEC];
+                // x row u of the wave as the conv saw it (h when gated)
+                auto read_x = [&](int u, float (&xv)[VEC]) {
+                    if constexpr (GATED) {
+                        float uu[VEC], gg[VEC];
+                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, uu);
+                        lds_read_row<BF16, VEC>(lpx + XT_BYTES + u * SH::CB_BYTES, gg);
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) {
+                            const float sg = sigmoid_f32(gg[v]);
+                            gs[u][v] = gg[v] * sg;
+                            gd[u][v] = uu[v] * sg * (1.f + gg[v] * (1.f - sg));
+                            xv[v] = uu[v] * gs[u][v];
+                        }
+                    } else {
+                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                    }
+                };
+                // write the wave's dx rows (du and dg rows of dz when gated) from the conv's input gradient
+                auto emit_dx = [&](float (&acc)[WDX ? RW : 1][VEC]) {
+                    if constexpr (WDX) {
+                        const int xrowb = (int)x_row_bytes;
+                        if constexpr (GATED) {
+#pragma unroll
+                            for (int u = 0; u < RW; ++u) {
+                                float du[VEC], dg[VEC];
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    du[v] = acc[u][v] * gs[u][v];
+                                    dg[v] = acc[u][v] * gd[u][v];
+                                }
+                                Row ou, og;
+                                ou.from_f32(du);
+                                og.from_f32(dg);
+                                if (active && tf + u < T) {
+                                    ou.bstore(ro, out_voff, u * xrowb);
+                                    og.bstore(ro, out_voff + rowb, u * xrowb);
+                                }
+                            }
+                        } else {
+                            Row o[RW];
+#pragma unroll
+                            for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                            if (active) {
+#pragma unroll
+                                for (int u = 0; u < RW; ++u)
+                                    if (tf + u < T) o[u].bstore(ro, out_voff, u * xrowb);
+                            }
+                        }
+                    }
+                };
                 if (interior) {
                     float xc[WDW ? RW : 1][VEC];
                     if constexpr (WDW) {
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
-                            lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
+                            read_x(u, xc[u]);
                             if (tf + u >= T) {     // rows past the end contribute nothing
 #pragma unroll
                                 for (int v = 0; v < VEC; ++v) xc[u][v] = 0.f;
@@ -456,16 +553,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             }
                         }
                     }
-                    if constexpr (WDX) {
-                        Row o[RW];
-#pragma unroll
-                        for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
-                        if (active) {
-#pragma unroll
-                            for (int u = 0; u < RW; ++u)
-                                if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
-                        }
-                    }
+                    emit_dx(acc);
                 } else {
                     // A sequence boundary falls inside the wave's window: same unrolled schedule, every
                     // tap selected (never multiplied by 0) by bit m of its output row's tap mask.
@@ -474,7 +562,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     float xc[WDW ? RW : 1][VEC];
                     if constexpr (WDW) {
 #pragma unroll
-                        for (int u = 0; u < RW; ++u) lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xc[u]);
+                        for (int u = 0; u < RW; ++u) read_x(u, xc[u]);
                     }
                     float acc[WDX ? RW : 1][VEC];
                     if constexpr (WDX) {
@@ -523,16 +611,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             for (int v = 0; v < VEC; ++v) pin_regs<K>(dwa[v]);
                         }
                     }
-                    if constexpr (WDX) {
-                        Row o[RW];
-#pragma unroll
-                        for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
-                        if (active) {
-#pragma unroll
-                            for (int u = 0; u < RW; ++u)
-                                if (tf + u < T) o[u].bstore(ro, out_voff, u * rowb);
-                        }
-                    }
+                    emit_dx(acc);
                 }
             }
             if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, cu, S, T, t0 + g.nbt * R + rg * RW);

@@ -1,0 +1,124 @@
+"""Gated depthwise conv: ``conv(x_proj * silu(gate))`` with the gate product fused into the kernels.
+
+For a conv placed inside the reference's SwiGLU MLP
+(src/nanoplm/pretraining/models/modern_bert/modeling.py:300-302)::
+
+    x_proj, gate = self.Wi(x).chunk(2, dim=-1)
+    h = F.silu(gate) * x_proj            # [T, intermediate]
+    h = conv(h, cu_seqlens)              # <- here
+    return self.Wo(self.drop(h))
+
+``gated_varlen_dwconv(z, cu_seqlens, weight, bias)`` takes ``z = self.Wi(x)`` (``[T, 2C]``: x_proj in
+columns ``[0, C)``, gate in ``[C, 2C)``) and returns ``conv(h)`` ``[T, C]`` without ever writing ``h``:
+the forward reads z once and writes y, the backward reads z and dy and writes dz = [d x_proj | d gate],
+dw and db. Shapes the fused kernels are not built for (see ``gated_supported``) run the same HIP
+conv after the gate product is formed with ordinary elementwise ops.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from . import _lib
+from .dwconv import _DTYPES, _ptr, varlen_dwconv
+
+
+def gated_supported(z: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the fused kernels take this call (kernel size 3/5/7/9, rows of C*elemsize >= 1 KiB in
+    multiples of 16 bytes, 16-byte aligned contiguous z on a ROCm device)."""
+    if not (isinstance(z, torch.Tensor) and z.is_cuda and z.dim() == 2 and z.shape[1] % 2 == 0):
+        return False
+    if z.dtype not in _DTYPES or weight.dtype not in _DTYPES or not z.is_contiguous() or z.data_ptr() % 16:
+        return False
+    T, C2 = z.shape
+    K = weight.shape[1]
+    return int(_lib.load().nplm_dwconv_gated_bwd_workspace_bytes(max(T, 1), C2 // 2, K, _DTYPES[z.dtype])) > 0
+
+
+def _check(z, cu_seqlens, weight, bias):
+    if z.dim() != 2 or z.shape[1] % 2:
+        raise ValueError("z must be [T, 2C]: x_proj columns followed by gate columns")
+    T, C = z.shape[0], z.shape[1] // 2
+    if tuple(weight.shape[:1]) != (C,) or weight.dim() != 2:
+        raise ValueError(f"weight must be [C={C}, K], got {tuple(weight.shape)}")
+    if bias is not None and tuple(bias.shape) != (C,):
+        raise ValueError(f"bias must be [C={C}], got {tuple(bias.shape)}")
+    if cu_seqlens.dtype != torch.int32 or cu_seqlens.dim() != 1 or cu_seqlens.numel() < 1:
+        raise TypeError("cu_seqlens must be a 1-D int32 tensor with at least one entry")
+    return T, C, weight.shape[1], cu_seqlens.numel() - 1
+
+
+def gated_dwconv_fwd(z, cu_seqlens, weight, bias=None, *, residual: bool = False):
+    """Raw fused forward (no autograd): y [T, C] = conv(z[:, :C] * silu(z[:, C:]))."""
+    T, C, K, S = _check(z, cu_seqlens, weight, bias)
+    lib = _lib.load()
+    z = z.contiguous()
+    weight = weight.contiguous()
+    if bias is not None:
+        bias = bias.to(weight.dtype).contiguous()
+    y = torch.empty((T, C), dtype=z.dtype, device=z.device)
+    with torch.cuda.device(z.device):
+        rc = lib.nplm_dwconv_gated_fwd(_ptr(z), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(bias), _ptr(y), T, C, K, S,
+                                       _DTYPES[z.dtype], _DTYPES[weight.dtype], _lib.RESIDUAL if residual else 0,
+                                       torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "nplm_dwconv_gated_fwd")
+    return y
+
+
+def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
+    """Raw fused backward: (dz [T, 2C] in z's dtype, dw [C, K] fp32, db [C] fp32)."""
+    T, C, K, S = _check(z, cu_seqlens, weight, None)
+    if tuple(dy.shape) != (T, C) or dy.dtype != z.dtype or dy.device != z.device:
+        raise ValueError("dy must be [T, C] in z's dtype on z's device")
+    lib = _lib.load()
+    z = z.contiguous()
+    dy = dy.contiguous()
+    weight = weight.contiguous()
+    act = _DTYPES[z.dtype]
+    dz = torch.empty_like(z)
+    dw = torch.empty((C, K), dtype=torch.float32, device=z.device)
+    db = torch.empty((C,), dtype=torch.float32, device=z.device)
+    with torch.cuda.device(z.device):
+        nbytes = int(lib.nplm_dwconv_gated_bwd_workspace_bytes(T, C, K, act))
+        ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=z.device)
+        rc = lib.nplm_dwconv_gated_bwd(_ptr(z), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(dz), _ptr(dw),
+                                       _ptr(db), _ptr(ws), ws.numel(), T, C, K, S, act, _DTYPES[weight.dtype],
+                                       _lib.RESIDUAL if residual else 0, torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "nplm_dwconv_gated_bwd")
+    return dz, dw, db
+
+
+class GatedVarlenDWConv1dFunction(torch.autograd.Function):
+    """``apply(z, cu_seqlens, weight, bias, residual) -> y``; backward returns ``(dz, None, dw, db, None)``."""
+
+    @staticmethod
+    def forward(ctx, z, cu_seqlens, weight, bias=None, residual=False):
+        y = gated_dwconv_fwd(z, cu_seqlens, weight, bias, residual=bool(residual))
+        ctx.save_for_backward(z, cu_seqlens, weight)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        ctx.residual = bool(residual)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        z, cu_seqlens, weight = ctx.saved_tensors
+        if dy.dtype != z.dtype:
+            dy = dy.to(z.dtype)
+        dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=ctx.residual)
+        return (dz if ctx.needs_input_grad[0] else None, None,
+                dw.to(weight.dtype) if ctx.needs_input_grad[2] else None,
+                db.to(ctx.bias_dtype) if (ctx.bias_dtype is not None and ctx.needs_input_grad[3]) else None, None)
+
+
+def gated_varlen_dwconv(z: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
+                        bias: Optional[torch.Tensor] = None, residual: bool = False) -> torch.Tensor:
+    """``conv(z[:, :C] * silu(z[:, C:]))`` over packed sequences, ``[T, 2C] -> [T, C]``.
+
+    Fused kernels where they are built (``gated_supported``); otherwise the gate product is formed by
+    elementwise ops and the plain HIP conv runs on it (same result to rounding)."""
+    if gated_supported(z, weight):
+        return GatedVarlenDWConv1dFunction.apply(z, cu_seqlens, weight, bias, residual)
+    x_proj, gate = z.chunk(2, dim=-1)
+    return varlen_dwconv((F.silu(gate) * x_proj).contiguous(), cu_seqlens, weight, bias, residual)

@@ -72,6 +72,22 @@ def ref_dwconv_varlen_grads(x, cu_seqlens, weight, bias, dy, compute_dtype=torch
     return y.detach(), xr.grad, wr.grad, db
 
 
+def ref_gated_dwconv_grads(z, cu_seqlens, weight, bias, dy, compute_dtype=torch.float64, residual=False):
+    """(y, dz, dw, db) of the reference MLP's gate product followed by the conv loop:
+    ``x_proj, gate = z.chunk(2, -1); h = F.silu(gate) * x_proj`` (modeling.py:300-302), then
+    ``ref_dwconv_varlen(h)``, gradients by autograd, everything in ``compute_dtype``."""
+    zr = z.detach().to(compute_dtype).requires_grad_(True)
+    wr = weight.detach().to(compute_dtype).requires_grad_(True)
+    br = None if bias is None else bias.detach().to(compute_dtype).requires_grad_(True)
+    x_proj, gate = zr.chunk(2, dim=-1)
+    h = F.silu(gate) * x_proj
+    y = ref_dwconv_varlen(h, cu_seqlens, wr, br, compute_dtype, residual)
+    if dy is None:
+        return y.detach()
+    y.backward(dy.to(compute_dtype))
+    return y.detach(), zr.grad, wr.grad, (None if br is None else br.grad)
+
+
 # --------------------------------------------------------------------------------------------
 # C oracle (definition, double accumulation)
 # --------------------------------------------------------------------------------------------

@@ -1,0 +1,99 @@
+"""Gated conv (conv over x_proj * silu(gate), the SwiGLU product of modeling.py:300-302, fused into the
+kernels) against the float64 oracle, through the C ABI entry points and the autograd surface."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+import nanoplm_amd as npa
+from nanoplm_amd import _lib
+from nanoplm_amd.workloads import cu_from_lengths, make_workload
+from oracle import dwconv_ref as O
+from tests.gpu_util import assert_act_close, assert_red_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+LENS_MIX = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 17, 512]
+
+
+def _case(lens, C, K, dt, wdt, seed):
+    g = torch.Generator().manual_seed(seed)
+    T = int(sum(lens))
+    z = torch.randn(T, 2 * C, generator=g).to(dt)
+    w = (torch.randn(C, K, generator=g) * K ** -0.5).to(wdt)
+    b = (torch.randn(C, generator=g) * 0.02).to(wdt)
+    dy = torch.randn(T, C, generator=g).to(dt)
+    return z, cu_from_lengths(torch.tensor(lens)), w, b, dy
+
+
+def _check(z, cu, w, b, dy, what, residual=False):
+    y64, dz64, dw64, db64 = O.ref_gated_dwconv_grads(z, cu, w, b, dy, torch.float64, residual)
+    zd, cud, wd, bd, dyd = (t.to(DEV) for t in (z, cu, w, b, dy))
+    assert npa.gated_supported(zd, wd)
+    y = npa.gated_dwconv_fwd(zd, cud, wd, bd, residual=residual)
+    dz, dw, db = npa.gated_dwconv_bwd(zd, dyd, cud, wd, residual=residual)
+    assert y.shape == dy.shape and dz.shape == z.shape
+    assert_act_close(y, y64, z.dtype, what + " y")
+    assert_act_close(dz, dz64, z.dtype, what + " dz")
+    assert_red_close(dw, dw64, what + " dw")
+    assert_red_close(db, db64, what + " db")
+
+
+@pytest.mark.parametrize("K", [3, 5, 7, 9])
+@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.bfloat16, 520), (torch.float32, 256), (torch.float32, 768)])
+def test_gated_kernel_sizes_and_widths(K, dt, C):
+    print(f"[case] gated K={K} C={C} {dt}", flush=True)
+    _check(*_case(LENS_MIX, C, K, dt, dt, seed=K + C), f"gated K={K} C={C} {dt}")
+
+
+def test_gated_intermediate_width_with_fp32_weights_and_residual():
+    _check(*_case(LENS_MIX, 2048, 7, torch.bfloat16, torch.float32, seed=4), "gated C=2048 bf16/fp32")
+    _check(*_case(LENS_MIX, 1024, 7, torch.bfloat16, torch.bfloat16, seed=6), "gated residual", residual=True)
+
+
+def test_gated_boundary_stress_and_partial_last_tile():
+    wl = make_workload(5, T=20011, C=1024, with_dy=True)        # lengths of 1..8 mixed with 400..512, odd T
+    g = torch.Generator().manual_seed(9)
+    z = torch.randn(wl.T, 2048, generator=g).bfloat16()
+    _check(z, wl.cu_seqlens, wl.weight, wl.bias, wl.dy, "gated boundary stress")
+
+
+def test_gated_autograd_matches_the_unfused_composition_and_is_deterministic():
+    z, cu, w, b, dy = _case(LENS_MIX, 1024, 7, torch.float32, torch.float32, seed=12)
+    cud, dyd = cu.to(DEV), dy.to(DEV)
+    z1 = z.to(DEV).requires_grad_(True)
+    w1 = w.to(DEV).requires_grad_(True)
+    b1 = b.to(DEV).requires_grad_(True)
+    y1 = npa.gated_varlen_dwconv(z1, cud, w1, b1)
+    y1.backward(dyd)
+    z2 = z.to(DEV).requires_grad_(True)
+    w2 = w.to(DEV).requires_grad_(True)
+    b2 = b.to(DEV).requires_grad_(True)
+    u, g = z2.chunk(2, dim=-1)
+    y2 = npa.varlen_dwconv((F.silu(g) * u).contiguous(), cud, w2, b2)
+    y2.backward(dyd)
+    torch.testing.assert_close(y1, y2, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(z1.grad, z2.grad, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(w1.grad, w2.grad, rtol=1e-5, atol=1e-3)
+    torch.testing.assert_close(b1.grad, b2.grad, rtol=1e-5, atol=1e-3)
+    # second run: bit-identical
+    z3 = z.to(DEV).requires_grad_(True)
+    w3 = w.to(DEV).requires_grad_(True)
+    y3 = npa.gated_varlen_dwconv(z3, cud, w3, b.to(DEV))
+    y3.backward(dyd)
+    assert torch.equal(y3, y1) and torch.equal(z3.grad, z1.grad) and torch.equal(w3.grad, w1.grad)
+
+
+def test_unsupported_shapes_compose_and_the_abi_says_so():
+    z, cu, w, b, dy = _case([5, 40, 3], 100, 7, torch.bfloat16, torch.bfloat16, seed=1)     # 200-byte rows
+    zd, cud, wd, bd = z.to(DEV), cu.to(DEV), w.to(DEV), b.to(DEV)
+    assert not npa.gated_supported(zd, wd)
+    y = npa.gated_varlen_dwconv(zd, cud, wd, bd)
+    y64 = O.ref_gated_dwconv_grads(z, cu, w, b, None)
+    assert float((y.cpu().double() - y64).abs().max()) <= 3e-2      # h is rounded to bf16 on this route
+    lib = _lib.load()
+    out = torch.empty(48, 100, device=DEV, dtype=torch.bfloat16)
+    rc = lib.nplm_dwconv_gated_fwd(zd.data_ptr(), cud.data_ptr(), wd.data_ptr(), None, out.data_ptr(), 48, 100, 7, 3, 1, 1, 0,
+                                   torch.cuda.current_stream().cuda_stream)
+    assert rc == -_lib.EUNSUPPORTED and "gated" in _lib.strerror(rc)
+    z11, _, w11, b11, _ = _case([30, 30], 1024, 11, torch.bfloat16, torch.bfloat16, seed=2)  # K = 11
+    assert not npa.gated_supported(z11.to(DEV), w11.to(DEV))

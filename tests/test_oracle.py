@@ -299,3 +299,46 @@ def test_residual_oracles_agree_and_reduce_to_the_centre_weight_identity():
     # w = 0, b = 0: the identity
     y0 = O.ref_dwconv_varlen(x, cu, torch.zeros_like(w), None, torch.float64, residual=True)
     assert torch.equal(y0, x)
+
+
+# ---- gated input (x_proj * silu(gate)) -------------------------------------------------------------------
+def test_gated_oracle_against_closed_forms_and_finite_differences():
+    """h = x_proj * gate / (1 + exp(-gate)) written out with numpy; gate = 0 silences the input (y = b);
+    a large gate passes gate * x_proj through; dz against central differences in float64."""
+    import numpy as np
+    g = torch.Generator().manual_seed(5)
+    lens = torch.tensor([4, 1, 9, 2])
+    cu = torch.zeros(len(lens) + 1, dtype=torch.int32)
+    cu[1:] = torch.cumsum(lens, 0)
+    T, C, K = int(lens.sum()), 3, 5
+    z = torch.randn(T, 2 * C, generator=g, dtype=torch.float64)
+    w = torch.randn(C, K, generator=g, dtype=torch.float64)
+    b = torch.randn(C, generator=g, dtype=torch.float64)
+    dy = torch.randn(T, C, generator=g, dtype=torch.float64)
+    y, dz, dw, db = O.ref_gated_dwconv_grads(z, cu, w, b, dy)
+    zn = z.numpy()
+    h = torch.from_numpy(zn[:, :C] * zn[:, C:] / (1.0 + np.exp(-zn[:, C:])))
+    yb, dhb, dwb, dbb = O.brute_force(h, cu, w, b, dy)
+    torch.testing.assert_close(y, yb, rtol=0, atol=1e-12)
+    torch.testing.assert_close(dw, dwb, rtol=0, atol=1e-12)
+    torch.testing.assert_close(db, dbb, rtol=0, atol=1e-12)
+    # chain rule by hand: d x_proj = dh * silu(g), d gate = dh * x_proj * sig * (1 + g (1 - sig))
+    sig = 1.0 / (1.0 + np.exp(-zn[:, C:]))
+    dzb = np.concatenate([dhb.numpy() * zn[:, C:] * sig, dhb.numpy() * zn[:, :C] * sig * (1 + zn[:, C:] * (1 - sig))], 1)
+    torch.testing.assert_close(dz, torch.from_numpy(dzb), rtol=0, atol=1e-12)
+    # central differences on a few entries of z
+    eps = 1e-6
+    for (t, c) in [(0, 0), (5, 4), (13, 2), (15, 5)]:
+        zp, zm = z.clone(), z.clone()
+        zp[t, c] += eps
+        zm[t, c] -= eps
+        fd = ((O.ref_gated_dwconv_grads(zp, cu, w, b, None) - O.ref_gated_dwconv_grads(zm, cu, w, b, None)) * dy).sum() / (2 * eps)
+        assert abs(float(fd) - float(dz[t, c])) < 1e-6
+    # gate = 0 -> h = 0 -> y = bias;  gate = 40 -> silu(gate) = gate to 1e-16
+    z0 = z.clone()
+    z0[:, C:] = 0
+    assert torch.equal(O.ref_gated_dwconv_grads(z0, cu, w, b, None), b.expand(T, C))
+    z1 = z.clone()
+    z1[:, C:] = 40.0
+    torch.testing.assert_close(O.ref_gated_dwconv_grads(z1, cu, w, b, None), O.ref_dwconv_varlen(40.0 * z[:, :C], cu, w, b, torch.float64),
+                               rtol=1e-14, atol=1e-12)
