@@ -21,7 +21,9 @@ from .padded import (  # noqa: F401
 from .gated import (  # noqa: F401
     GatedVarlenDWConv1dFunction,
     gated_dwconv_bwd,
+    gated_dwconv_bwd_op,
     gated_dwconv_fwd,
+    gated_dwconv_fwd_op,
     gated_supported,
     gated_varlen_dwconv,
 )

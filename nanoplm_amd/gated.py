@@ -118,7 +118,60 @@ def gated_varlen_dwconv(z: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch
 
     Fused kernels where they are built (``gated_supported``); otherwise the gate product is formed by
     elementwise ops and the plain HIP conv runs on it (same result to rounding)."""
-    if gated_supported(z, weight):
+    if torch.compiler.is_compiling():
+        # static shapes under torch.compile: a contiguous [T, 2C] activation of a supported width takes the
+        # registered fused ops (opaque to the tracer, no graph break)
+        if z.dim() == 2 and z.is_contiguous() and weight.shape[1] in (3, 5, 7, 9) and \
+                (z.shape[1] // 2 * z.element_size()) % 16 == 0 and z.shape[1] // 2 * z.element_size() >= 1024:
+            return gated_dwconv_fwd_op(z, cu_seqlens, weight, bias, residual)
+    elif gated_supported(z, weight):
         return GatedVarlenDWConv1dFunction.apply(z, cu_seqlens, weight, bias, residual)
     x_proj, gate = z.chunk(2, dim=-1)
     return varlen_dwconv((F.silu(gate) * x_proj).contiguous(), cu_seqlens, weight, bias, residual)
+
+
+# ---------------------------------------------------------------------------------------------
+# torch.library registration of the fused pair, so that a compiled model
+# (torch.compile(dynamic=False), src/nanoplm/pretraining/pure_pipeline.py:519-524) keeps one graph.
+# ---------------------------------------------------------------------------------------------
+@torch.library.custom_op("nanoplm_amd::gated_dwconv_fwd", mutates_args=(), device_types="cuda")
+def gated_dwconv_fwd_op(z: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
+                        bias: Optional[torch.Tensor], residual: bool = False) -> torch.Tensor:
+    return gated_dwconv_fwd(z, cu_seqlens, weight, bias, residual=residual)
+
+
+@gated_dwconv_fwd_op.register_fake
+def _(z, cu_seqlens, weight, bias, residual=False):
+    return z.new_empty((z.shape[0], z.shape[1] // 2))
+
+
+@torch.library.custom_op("nanoplm_amd::gated_dwconv_bwd", mutates_args=(), device_types="cuda")
+def gated_dwconv_bwd_op(z: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
+                        residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=residual)
+    return dz, dw, db
+
+
+@gated_dwconv_bwd_op.register_fake
+def _(z, dy, cu_seqlens, weight, residual=False):
+    C, K = weight.shape
+    return (torch.empty_like(z, memory_format=torch.contiguous_format),
+            z.new_empty((C, K), dtype=torch.float32), z.new_empty((C,), dtype=torch.float32))
+
+
+def _gated_setup_context(ctx, inputs, output):
+    z, cu_seqlens, weight, bias, residual = inputs
+    ctx.save_for_backward(z, cu_seqlens, weight)
+    ctx.bias_dtype = None if bias is None else bias.dtype
+    ctx.residual = bool(residual)
+
+
+def _gated_backward(ctx, dy):
+    z, cu_seqlens, weight = ctx.saved_tensors
+    if dy.dtype != z.dtype:
+        dy = dy.to(z.dtype)
+    dz, dw, db = gated_dwconv_bwd_op(z, dy.contiguous(), cu_seqlens, weight, ctx.residual)
+    return dz, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype)), None
+
+
+gated_dwconv_fwd_op.register_autograd(_gated_backward, setup_context=_gated_setup_context)

@@ -97,3 +97,29 @@ def test_unsupported_shapes_compose_and_the_abi_says_so():
     assert rc == -_lib.EUNSUPPORTED and "gated" in _lib.strerror(rc)
     z11, _, w11, b11, _ = _case([30, 30], 1024, 11, torch.bfloat16, torch.bfloat16, seed=2)  # K = 11
     assert not npa.gated_supported(z11.to(DEV), w11.to(DEV))
+
+
+def test_gated_ops_pass_opcheck_and_compile_without_graph_breaks():
+    z, cu, w, b, dy = _case([40, 3, 200, 13], 1024, 7, torch.bfloat16, torch.bfloat16, seed=21)
+    zd, cud, wd, bd, dyd = (t.to(DEV) for t in (z, cu, w, b, dy))
+    torch.library.opcheck(npa.gated_dwconv_fwd_op, (zd, cud, wd, bd), test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(npa.gated_dwconv_bwd_op, (zd, dyd, cud, wd), test_utils=("test_schema", "test_faketensor"))
+
+    class MLPTail(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = npa.VarlenDWConv1d(1024, 7, device=DEV, dtype=torch.bfloat16)
+
+        def forward(self, zz, cc):
+            return npa.gated_varlen_dwconv(zz, cc, self.conv.weight, self.conv.bias)
+
+    m = MLPTail()
+    z1 = zd.clone().requires_grad_(True)
+    eager = m(z1, cud)
+    eager.backward(dyd)
+    compiled = torch.compile(m, backend="aot_eager", fullgraph=True, dynamic=False)
+    z2 = zd.clone().requires_grad_(True)
+    m.zero_grad()
+    out = compiled(z2, cud)
+    out.backward(dyd)
+    assert torch.equal(out, eager) and torch.equal(z2.grad, z1.grad)
