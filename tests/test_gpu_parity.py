@@ -303,3 +303,34 @@ def test_linearity_and_adjoint_identity_at_full_size():
     assert torch.equal(y2, y * 2)
     _, dw2, _ = npa.varlen_dwconv_bwd(x * 2, dy, cu, w, need_dx=False)
     assert torch.equal(dw2, dw * 2)
+
+
+def test_rows_beyond_2_and_4_gib_offsets():
+    """Maximum-size edge: 2.2 M rows x 2 KiB = 4.5 GB per tensor, so row offsets cross both 2^31 and 2^32
+    bytes. Size-independent property: a run of whole sequences cut out of the big batch and processed
+    alone (re-based cu_seqlens) gives bit-identical y and dx; dw/db agree between the two kernel families."""
+    T, C, K = 2_200_000, 1024, 7
+    g = torch.Generator().manual_seed(77)
+    lens = torch.randint(20, 513, (T // 200,), generator=g)
+    lens = lens[torch.cumsum(lens, 0) <= T]
+    lens = torch.cat([lens, torch.tensor([T - int(lens.sum())])])
+    cu = cu_from_lengths(lens).to(DEV)
+    x = torch.randn(T, C, device=DEV, dtype=torch.bfloat16)
+    dy = torch.randn(T, C, device=DEV, dtype=torch.bfloat16)
+    w = (torch.randn(C, K, device=DEV) * K ** -0.5).bfloat16()
+    b = (torch.randn(C, device=DEV) * 0.02).bfloat16()
+    y = npa.varlen_dwconv_fwd(x, cu, w, b)
+    dx, dw, db = npa.varlen_dwconv_bwd(x, dy, cu, w)
+    cul = cu.tolist()
+    S = len(cul) - 1
+    for first, count in ((0, 40), (S // 2 - 20, 40), (S - 40, 40)):     # start, around 2-4 GiB, end
+        s, e = cul[first], cul[first + count]
+        sub = (cu[first:first + count + 1] - s).contiguous()
+        ys = npa.varlen_dwconv_fwd(x[s:e], sub, w, b)
+        dxs, _, _ = npa.varlen_dwconv_bwd(x[s:e], dy[s:e], sub, w)
+        assert torch.equal(y[s:e], ys) and torch.equal(dx[s:e], dxs), f"rows {s}..{e}"
+    assert (S // 2) > 0 and cul[S // 2] * C * 2 > 2 ** 31 and cul[S - 40] * C * 2 > 2 ** 32
+    _, dw1, db1 = npa.varlen_dwconv_bwd(x, dy, cu, w, need_dx=False, tuning=_lib.Tuning(algo=1))
+    torch.testing.assert_close(dw, dw1, rtol=2e-5, atol=0.05)
+    torch.testing.assert_close(db, db1, rtol=2e-5, atol=0.05)
+    torch.testing.assert_close(db, dy.float().sum(0), rtol=2e-5, atol=0.05)
