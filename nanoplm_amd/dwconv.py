@@ -252,6 +252,12 @@ class VarlenDWConv1d(nn.Module):
             return varlen_dwconv_fwd_op(x, cu_seqlens, self.weight, self.bias, self.residual)
         return VarlenDWConv1dFunction.apply(x, cu_seqlens, self.weight, self.bias, self.residual)
 
+    def forward_gated(self, z: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
+        """SwiGLU door: ``z = Wi(x)`` of width ``2 * channels`` (x_proj columns, then gate columns);
+        returns ``conv(x_proj * silu(gate))`` with the gate product fused into the kernels (see nanoplm_amd.gated)."""
+        from .gated import gated_varlen_dwconv
+        return gated_varlen_dwconv(z, cu_seqlens, self.weight, self.bias, self.residual)
+
     def extra_repr(self) -> str:
         return (f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}, "
                 f"residual={self.residual}, flat_weight={self.flat_weight}, init={self.init}")

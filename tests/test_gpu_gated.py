@@ -111,7 +111,7 @@ def test_gated_ops_pass_opcheck_and_compile_without_graph_breaks():
             self.conv = npa.VarlenDWConv1d(1024, 7, device=DEV, dtype=torch.bfloat16)
 
         def forward(self, zz, cc):
-            return npa.gated_varlen_dwconv(zz, cc, self.conv.weight, self.conv.bias)
+            return self.conv.forward_gated(zz, cc)
 
     m = MLPTail()
     z1 = zd.clone().requires_grad_(True)
