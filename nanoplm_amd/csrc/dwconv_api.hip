@@ -156,7 +156,7 @@ constexpr size_t kLdsBytesPerCU = 160u << 10;
 
 struct LdsPlan {
     LdsShapeSel sh;
-    int R, ntiles, ncb, nbt, xcd_group;
+    int R, ntiles, ncb, nbt, xcd_group, rot_step;
 };
 
 // Whether the LDS kernels can take this problem at all (16-byte row granularity, built kernel size).
@@ -221,6 +221,10 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     const long long nblocks = (long long)p.ncb * p.nbt;
     if (G > 0 && !(nblocks % kNumXCD == 0 && (nblocks / kNumXCD) % G == 0 && p.nbt % G == 0)) G = 0;
     p.xcd_group = G;
+    // per-round rotation of the tile slots: an odd step near nbt / golden ratio, so that no short period of
+    // sequence boundaries keeps landing on the same token-blocks
+    p.rot_step = nbt > 2 ? (int)((long long)nbt * 618 / 1000) | 1 : 0;
+    if (p.rot_step >= nbt) p.rot_step = nbt - 1;
     *out = p;
     return 0;
 }
@@ -228,7 +232,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
 LdsGeo make_lds_geo(const LdsPlan& p, long long T, int C, int S, int w_flags) {
     LdsGeo g{};
     g.T = (int32_t)T; g.C = C; g.S = S; g.w_flags = w_flags;
-    g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_group = p.xcd_group;
+    g.ntiles = p.ntiles; g.ncb = p.ncb; g.nbt = p.nbt; g.xcd_group = p.xcd_group; g.rot_step = p.rot_step;
     return g;
 }
 

@@ -14,8 +14,8 @@
 //
 // The two tiles live in two LDS buffers; one workgroup barrier per tile hands the freshly loaded
 // buffer to the compute waves and the consumed one back to the loaders, so HBM traffic and
-// arithmetic overlap inside one block. Blocks walk tiles grid-stride (tile, tile + nbt, ...): all
-// resident blocks together sweep one compact window of rows, the access pattern HBM serves fastest,
+// arithmetic overlap inside one block. Blocks walk tiles in rounds of nbt (one tile per block and
+// round): all resident blocks together sweep one compact window of rows, the access pattern HBM serves fastest,
 // and the halo rows a block re-reads were fetched moments earlier by its neighbour.
 //
 // Backward: x and dy tiles are staged the same way; dx is written per tile, dw/db stay in registers
@@ -23,11 +23,16 @@
 // through LDS in fixed order, one slab per token-block, then dwconv_finalize_kernel). No atomics.
 //
 // Sequence boundaries: the cursor lookup for the NEXT tile (a chain of dependent scalar loads) runs
-// right before the tile barrier, where the compute waves would otherwise idle. A wave whose rows and
-// taps all lie in one sequence takes an unmasked path. A wave that touches a boundary keeps the
-// same unrolled schedule and selects every tap by a bit of its output row's tap mask; that path
-// must stay close to the unmasked one in cost, because tiles are dealt to blocks statically and a
-// block's time is the sum of its tiles: a slow boundary path shows up as a long tail of the grid.
+// where it costs least: in the forward on the loader waves, which idle while their loads are in
+// flight and post the result in a small LDS mailbox (the forward's compute waves are themselves
+// memory-bound through their stores); in the backward on the compute waves right before the tile
+// barrier. A wave whose rows and taps all lie in one sequence takes an unmasked path. A wave that
+// touches a boundary keeps the same unrolled schedule and selects every tap by a bit of its output
+// row's tap mask (K = 31: one unmasked pass per sequence over that sequence's rows); that path must
+// stay close to the unmasked one in cost, because tiles are dealt to blocks statically and a block's
+// time is the sum of its tiles: a slow boundary path shows up as a long tail of the grid. For the
+// same reason the tile slots rotate from round to round (lds_next_slot), so that boundaries at a
+// regular period do not pile up on a few blocks.
 //
 // Every wave of a block executes exactly the same sequence of barriers: the trip counts depend only
 // on blockIdx and the launch geometry.
@@ -45,6 +50,7 @@ struct LdsGeo {
     int32_t ntiles;     // ceil(T / R)
     int32_t ncb, nbt;   // grid = ncb column blocks x nbt token blocks (nbt <= ntiles)
     int32_t xcd_group;  // > 0: runs of this many adjacent token-blocks share an XCD (and its L2)
+    int32_t rot_step;   // per-round rotation of the tile slots, 0 <= rot_step < nbt
 };
 
 // blockIdx -> (column block, token block). Hardware deals consecutive workgroups round-robin to the
@@ -67,7 +73,29 @@ __device__ __forceinline__ void lds_block_coords(const LdsGeo& g, int& cb, int& 
     }
 }
 
+// Round r of the grid covers tiles r*nbt .. r*nbt + nbt-1, and token-block tb takes slot
+// (tb + r*rot_step) mod nbt of them. Tiles are dealt statically (dw/db must not depend on timing), and
+// without the rotation sequence boundaries that recur at a period dividing nbt tiles (equal-length
+// sequences, padded batches) would all fall to the same few blocks, whose slower boundary path then
+// becomes the tail of the whole grid. Adjacent token-blocks still take adjacent tiles (modulo the
+// wrap), so the XCD grouping above keeps its halo sharing. The slot is carried from round to round
+// (one add and a conditional subtract; rot_step < nbt).
+__device__ __forceinline__ int lds_next_slot(const LdsGeo& g, int q) {
+    q += g.rot_step;
+    return q >= g.nbt ? q - g.nbt : q;
+}
+// First row of the tile in slot q of round r; T when the slot lies past the last tile (last round
+// only): the block then idles through that round.
+__device__ __forceinline__ int lds_tile_row0(const LdsGeo& g, int r, int q, int R) {
+    const int tile = r * g.nbt + q;
+    return tile < g.ntiles ? tile * R : g.T;
+}
+
 typedef __attribute__((address_space(3))) void lds_void;
+
+// LDS a workgroup can have, and whether the forward's boundary mailbox fits behind `tile_bytes` of tiles.
+constexpr int kLdsBytes = 160 * 1024;
+constexpr bool lds_mail_fits(long long tile_bytes, int mail_bytes) { return tile_bytes + mail_bytes <= kLdsBytes; }
 
 // s_waitcnt vmcnt(0) (expcnt / lgkmcnt untouched), gfx9 encoding.
 __device__ __forceinline__ void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -85,6 +113,7 @@ struct LdsShape {
     static constexpr int CB_CH = NCW * 64 * VEC;        // channels in one column block
     static constexpr int NPIECE = CB_BYTES / 1024;      // 1 KiB direct loads per staged row
     static constexpr int TILE_BYTES = NROWS * CB_BYTES;
+    static constexpr int MAIL_BYTES = 2 * NRG * 16;     // forward: two sets of one 16-byte boundary record per row group
     static_assert(CB_BYTES % 1024 == 0, "a column block must be a whole number of 1 KiB wave loads");
     static_assert((NPIECE & (NPIECE - 1)) == 0, "pieces per row must be a power of two");
     static_assert(NROWS * CB_BYTES <= 65536, "ds_read immediate offsets are 16 bit");
@@ -168,13 +197,28 @@ __device__ __forceinline__ void lds_read_gated_row(const char* pu, const char* p
 // The expensive part of the boundary lookup: position the cursor on the sequence of row tf (a chain
 // of dependent scalar loads). The compute waves run it for the NEXT tile right before the tile
 // barrier, where they would otherwise idle until the loaders' data has landed.
-// Returns true when every tap of rows tf .. tf+RW-1 lies inside that one sequence.
+// Returns true when every tap of rows tf .. tf+RW-1 lies inside that one sequence. Otherwise `nce`
+// receives the end of the interval that follows the cursor's, so that crossing the (usually only)
+// boundary inside the wave's rows costs no scalar load in the middle of the tile's arithmetic.
 template <int RW, int P>
-__device__ __forceinline__ bool wave_locate(SeqCursor& sc, const int32_t* __restrict__ cu, int S, int T, int tf) {
+__device__ __forceinline__ bool wave_locate(SeqCursor& sc, int& nce, const int32_t* __restrict__ cu, int S, int T, int tf) {
     if (tf >= T) return true;
     sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
     const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
-    return (tf - P >= sc.cs) && (tl + P < sc.ce);
+    const bool in = (tf - P >= sc.cs) && (tl + P < sc.ce);
+    if (!in) nce = (sc.seq + 1 < S) ? cu_at(cu, sc.seq + 2) : T;
+    return in;
+}
+// SeqCursor::advance that takes its first step from the prefetched `nce` (valid while `fresh`).
+__device__ __forceinline__ void advance_prefetched(SeqCursor& sq, int nce, bool& fresh, const int32_t* __restrict__ cu,
+                                                   int S, int T, int t) {
+    if (fresh && t >= sq.ce && sq.seq < S) {
+        ++sq.seq;
+        sq.cs = sq.ce;
+        sq.ce = nce;
+        fresh = false;
+    }
+    sq.advance(cu, S, T, t);
 }
 
 // Empty volatile asm that takes N registers in and out: orders the instructions that produce them
@@ -187,16 +231,18 @@ __device__ __forceinline__ void pin_regs(float (&r)[N]) {
 
 // Tap masks of a wave's RW output rows, for a wave whose rows touch a sequence boundary: bit m of
 // vm[u] is set iff tap row (tf + u) - P + m lies inside the sequence of output row tf + u. Rows past
-// the end of the tensor get an empty mask. `sc` (by value) must be positioned on row tf.
+// the end of the tensor get an empty mask. `sc` (by value) must be positioned on row tf, `nce` is
+// what wave_locate left.
 template <int RW, int K>
-__device__ __forceinline__ void wave_tap_masks(SeqCursor sc, const int32_t* __restrict__ cu, int S, int T, int tf,
+__device__ __forceinline__ void wave_tap_masks(SeqCursor sc, int nce, const int32_t* __restrict__ cu, int S, int T, int tf,
                                                uint32_t (&vm)[RW]) {
+    bool fresh = true;
 #pragma unroll
     for (int u = 0; u < RW; ++u) {
         const int t = tf + u;
         uint32_t m = 0;
         if (t < T) {
-            sc.advance(cu, S, T, t);
+            advance_prefetched(sc, nce, fresh, cu, S, T, t);
             m = row_tap_mask<K>(sc, t);
         }
         vm[u] = m;
@@ -223,7 +269,13 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     constexpr int BUF_BYTES = SH::TILE_BYTES * (GATED ? 2 : 1);
     static_assert(NBUF == 2 || NBUF == 3, "two or three tile buffers");
     static_assert(!GATED || NBUF == 2, "the gated forward is double-buffered");
-    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x BUF_BYTES
+    // Where LDS has 32 bytes to spare per row group, the loader waves (idle while their loads are in
+    // flight) also run the boundary lookup for the next tile and leave the result in a mailbox behind
+    // the tile buffers; the compute waves, whose stores make them as memory-bound as the loaders, then
+    // pay one LDS read per tile instead of a chain of dependent scalar loads.
+    constexpr bool MAIL = lds_mail_fits((long long)NBUF * BUF_BYTES, SH::MAIL_BYTES);
+    extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x BUF_BYTES (+ MAIL_BYTES)
+    int4* box = reinterpret_cast<int4*>(lds_raw + NBUF * BUF_BYTES);  // [2][NRG] (cs, ce, nce, seq)
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
@@ -235,7 +287,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     const int rowb = (int)row_bytes;
     const int col_byte0 = cb * SH::CB_BYTES;
     const int valid_bytes = (rowb - col_byte0 < SH::CB_BYTES) ? rowb - col_byte0 : SH::CB_BYTES;
-    const int ntl = (g.ntiles - tb + g.nbt - 1) / g.nbt;   // tiles of this block (>= 1), same for all waves
+    const int ntl = (g.ntiles + g.nbt - 1) / g.nbt;        // rounds of the grid, the same for every block
     const size_t in_row_bytes = GATED ? 2 * row_bytes : row_bytes;   // pitch of x (z when gated)
     auto stage_tile = [&](char* buf, int first_row) {
         stage_rows_fixed<SH, CNT>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
@@ -259,10 +311,29 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     float bias[VEC];
 #pragma unroll
     for (int v = 0; v < VEC; ++v) bias[v] = 0.f;
+    SeqCursor sc;
+    sc.seq = 0; sc.cs = 0; sc.ce = 0;
+    // loader waves: locate the row groups of the tile that starts at row0 and post them in mailbox set `par`
+    // (a loader takes row groups lw, lw + NWL, ... in rising order, so its cursor only moves forward)
+    auto post_bounds = [&](int par, int row0) {
+        if constexpr (MAIL) {
+            for (int r = wv - SH::NWC; r < NRG; r += NWL) {
+                const int tf = row0 + r * RW;
+                int ne = 0;
+                if (tf < T) {
+                    sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
+                    ne = (sc.seq + 1 < S) ? cu_at(cu, sc.seq + 2) : T;
+                }
+                if (lane == 0) box[par * NRG + r] = make_int4(sc.cs, sc.ce, ne, sc.seq);
+            }
+        }
+    };
     if (is_loader) {
-        stage_tile(lds_raw, tb * R - P);
-        if (NBUF == 3 && ntl > 1) {
-            stage_tile(lds_raw + BUF_BYTES, (tb + g.nbt) * R - P);
+        stage_tile(lds_raw, tb * R - P);     // round 0: tile tb (< nbt <= ntiles)
+        post_bounds(0, tb * R);
+        const int r1 = ntl > 1 ? lds_tile_row0(g, 1, lds_next_slot(g, tb), R) : T;
+        if (NBUF == 3 && r1 < T) {
+            stage_tile(lds_raw + BUF_BYTES, r1 - P);
             wait_vmem_but<CNT>();     // tile 0 has landed, tile 1 may still be in flight
         } else {
             wait_vmem_all();
@@ -276,30 +347,42 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                                    : reinterpret_cast<const float*>(b)[c0 + v];
         }
     }
-    SeqCursor sc;
-    sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;               // bounds of the wave's rows in the tile about to be computed
-    if (!is_loader) interior = wave_locate<RW, P>(sc, cu, S, T, tb * R + rg * RW);
+    int nce = 0;                        // (not interior) end of the interval after the cursor's
+    if constexpr (!MAIL) {
+        if (!is_loader) interior = wave_locate<RW, P>(sc, nce, cu, S, T, tb * R + rg * RW);
+    }
     __syncthreads();
 
     int bcur = 0;                       // buffer of tile `it`
+    int q = tb;                         // the block's slot in round `it`
     for (int it = 0; it < ntl; ++it) {
-        const int t0 = (tb + it * g.nbt) * R;
+        const int t0 = lds_tile_row0(g, it, q, R);   // T when the block has no tile in the last round
+        const int qn = lds_next_slot(g, q);
         char* cur = lds_raw + bcur * BUF_BYTES;
         if (is_loader) {
-            // stage tile it + NBUF - 1 into the buffer freed by the barrier that ended iteration it - 1,
-            // then wait until tile it + 1 has landed
+            // stage the tile of round it + NBUF - 1 into the buffer freed by the barrier that ended round
+            // it - 1, then wait until the tile of round it + 1 has landed
             const int ahead = NBUF - 1;
-            if (it + ahead < ntl) {
+            const int rn = it + ahead < ntl ? lds_tile_row0(g, it + ahead, NBUF == 3 ? lds_next_slot(g, qn) : qn, R) : T;
+            if (rn < T) {
                 const int bnew = (bcur + ahead) % NBUF;
-                stage_tile(lds_raw + bnew * BUF_BYTES, t0 + ahead * g.nbt * R - P);
-                if (NBUF == 3) wait_vmem_but<CNT>(); else wait_vmem_all();
-            } else {
-                wait_vmem_all();
+                stage_tile(lds_raw + bnew * BUF_BYTES, rn - P);
             }
+            if (it + 1 < ntl) post_bounds((it + 1) & 1, lds_tile_row0(g, it + 1, qn, R));
+            if (NBUF == 3 && rn < T) wait_vmem_but<CNT>(); else wait_vmem_all();
         } else {
             const int tf = t0 + rg * RW;
             if (tf < T) {
+                if constexpr (MAIL) {
+                    const int4 m = box[(it & 1) * NRG + rg];
+                    sc.cs = __builtin_amdgcn_readfirstlane(m.x);
+                    sc.ce = __builtin_amdgcn_readfirstlane(m.y);
+                    nce = __builtin_amdgcn_readfirstlane(m.z);
+                    sc.seq = __builtin_amdgcn_readfirstlane(m.w);
+                    const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
+                    interior = (tf - P >= sc.cs) && (tl + P < sc.ce);
+                }
                 float acc[RW][VEC];
 #pragma unroll
                 for (int u = 0; u < RW; ++u)
@@ -320,9 +403,58 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                             }
                         }
                     }
+                } else if constexpr (K >= 15) {
+                    // Long kernels, a sequence boundary inside the wave's window: one pass per sequence that owns
+                    // output rows of the wave. A pass runs the unmasked schedule over the staged rows of
+                    // its sequence only (whole rows are skipped by scalar branches, nothing is multiplied
+                    // by zero) into a scratch set of accumulators, of which the sequence's own output
+                    // rows are kept. Every staged row is read in at most one pass, so the path costs
+                    // about what the unmasked one does, however many boundaries there are, and every
+                    // output row sums its taps in the same order as on the other paths (same bits).
+                    SeqCursor sq = sc;                      // positioned on row tf
+                    int u0 = 0;                             // first output row not yet produced
+                    bool fresh = true;
+                    while (u0 < RW && tf + u0 < T) {
+                        advance_prefetched(sq, nce, fresh, cu, S, T, tf + u0);
+                        // staged rows (j <-> global row tf - P + j) and output rows of this sequence
+                        int jlo = sq.cs - (tf - P), jhi = sq.ce - (tf - P), u1 = sq.ce - tf;
+                        jlo = __builtin_amdgcn_readfirstlane(jlo < 0 ? 0 : jlo);
+                        jhi = __builtin_amdgcn_readfirstlane(jhi > RW + K - 1 ? RW + K - 1 : jhi);
+                        u1 = __builtin_amdgcn_readfirstlane(u1 > RW ? RW : u1);
+                        float part[RW][VEC];
+#pragma unroll
+                        for (int u = 0; u < RW; ++u)
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) part[u][v] = bias[v];
+#pragma unroll
+                        for (int j = 0; j < RW + K - 1; ++j) {
+                            if (j >= jlo && j < jhi) {
+                                float xr[VEC];
+                                if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
+                                else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+#pragma unroll
+                                for (int u = 0; u < RW; ++u) {
+                                    if (j - u >= 0 && j - u < K) {
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v) part[u][v] = __builtin_fmaf(wr[v][j - u], xr[v], part[u][v]);
+                                    }
+                                }
+                            }
+                        }
+#pragma unroll
+                        for (int u = 0; u < RW; ++u) {
+                            if (u >= u0 && u < u1) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) acc[u][v] = part[u][v];
+                            }
+                        }
+                        u0 = u1;
+                    }
                 } else {
+                    // Short kernels: the unmasked schedule with every tap selected (never multiplied by
+                    // zero) by a bit of its output row's tap mask; cheaper than per-sequence passes here.
                     uint32_t vm[RW];
-                    wave_tap_masks<RW, K>(sc, cu, S, T, tf, vm);
+                    wave_tap_masks<RW, K>(sc, nce, cu, S, T, tf, vm);
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
@@ -351,10 +483,13 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         if (tf + u < T) o[u].bstore(ry, out_voff, u * rowb);
                 }
             }
-            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, cu, S, T, t0 + g.nbt * R + rg * RW);
+            if constexpr (!MAIL) {
+                if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+            }
         }
         __syncthreads();   // next tile is in LDS; this tile's buffer may be overwritten
         bcur = (bcur + 1 == NBUF) ? 0 : bcur + 1;
+        q = qn;
     }
 }
 
@@ -393,7 +528,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     const int rowb = (int)row_bytes;
     const int col_byte0 = cb * SH::CB_BYTES;
     const int valid_bytes = (rowb - col_byte0 < SH::CB_BYTES) ? rowb - col_byte0 : SH::CB_BYTES;
-    const int ntl = (g.ntiles - tb + g.nbt - 1) / g.nbt;
+    const int ntl = (g.ntiles + g.nbt - 1) / g.nbt;        // rounds of the grid, the same for every block
 
     const int wc = wv % NCW;
     const int rg = (wv / NCW) % NRG;
@@ -441,15 +576,19 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;
-    if (!is_loader) interior = wave_locate<RW, P>(sc, cu, S, T, tb * R + rg * RW);
+    int nce = 0;
+    if (!is_loader) interior = wave_locate<RW, P>(sc, nce, cu, S, T, tb * R + rg * RW);
     __syncthreads();
 
+    int q = tb;                         // the block's slot in round `it`
     for (int it = 0; it < ntl; ++it) {
-        const int t0 = (tb + it * g.nbt) * R;
+        const int t0 = lds_tile_row0(g, it, q, R);   // T when the block has no tile in the last round
+        const int qn = lds_next_slot(g, q);
         char* cur = lds_raw + (it & 1) * BUF_BYTES;
         if (is_loader) {
-            if (it + 1 < ntl) {
-                stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, t0 + g.nbt * R);
+            const int rn = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
+            if (rn < T) {
+                stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, rn);
                 wait_vmem_all();
             }
         } else {
@@ -558,7 +697,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     // A sequence boundary falls inside the wave's window: same unrolled schedule, every
                     // tap selected (never multiplied by 0) by bit m of its output row's tap mask.
                     uint32_t vm[RW];
-                    wave_tap_masks<RW, K>(sc, cu, S, T, tf, vm);
+                    wave_tap_masks<RW, K>(sc, nce, cu, S, T, tf, vm);
                     float xc[WDW ? RW : 1][VEC];
                     if constexpr (WDW) {
 #pragma unroll
@@ -614,9 +753,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     emit_dx(acc);
                 }
             }
-            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, cu, S, T, t0 + g.nbt * R + rg * RW);
+            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
         }
         __syncthreads();
+        q = qn;
     }
 
     if constexpr (!WDW) return;
