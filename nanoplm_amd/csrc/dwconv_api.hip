@@ -167,21 +167,23 @@ bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     return (long long)C * E >= 1024;
 }
 
-// Whether they are also the faster choice. A block always owns a 2 KiB column block (1 KiB at K = 31)
-// of its rows and the grid's time follows the number of column blocks, so a row that fills its
-// column blocks poorly wastes lanes and loader slots. Measured on MI355X (T=131072, K=7, bf16 rows
-// of 1024 .. 6144 bytes and fp32 rows of 1024 .. 3072 bytes): LDS-staged wins for a single column
-// block filled to 5/8 or more and for several filled to 4/5 or more on average; the sliding-window
-// kernels win otherwise (e.g. rows of 1024, 2560 and 3072 bytes).
+// Whether they are also the faster choice. A block owns one column block (2 KiB, 768 bytes for rows that
+// are a multiple of that, 1 KiB at K = 31) of its rows and the grid's time follows the number of column
+// blocks, so a row that fills its column blocks poorly wastes lanes and loader slots. Measured on MI355X
+// (T=131072, K=7, bf16 rows of 1024 .. 10240 bytes and fp32 rows of 1024 .. 8192 bytes): LDS-staged wins
+// for a single column block filled to 5/8 or more; for several, the backward needs them filled to 4/5
+// on average (rows of 2560 bytes: 260 against 215 us), the forward only to 11/20 (same rows: 143 against
+// 154 us); the sliding-window kernels win otherwise (e.g. rows of 1024 bytes).
 bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     if (!lds_eligible(bf16, T, C, K, align_bits)) return false;
     if (K > 9 && bwd) return false;        // K = 31: only the forward fits its registers
-    const LdsShapeSel sh = lds_default_shape(bwd, bf16, K);
     const long long E = bf16 ? 2 : 4;
-    const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
     const long long row_bytes = (long long)C * E;
+    const LdsShapeSel sh = lds_shape_for(bwd, bf16, K, row_bytes);
+    const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
     const long long ncb = ceil_div(row_bytes, cb_bytes);
-    return ncb == 1 ? row_bytes * 8 >= cb_bytes * 5 : row_bytes * 5 >= ncb * cb_bytes * 4;
+    if (ncb == 1) return row_bytes * 8 >= cb_bytes * 5;
+    return bwd ? row_bytes * 5 >= ncb * cb_bytes * 4 : row_bytes * 20 >= ncb * cb_bytes * 11;
 }
 
 int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out,
@@ -190,7 +192,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    p.sh = gated ? lds_gated_shape(bwd, bf16) : lds_default_shape(bwd, bf16, K);
+    p.sh = gated ? lds_gated_shape(bwd, bf16) : lds_shape_for(bwd, bf16, K, (long long)C * E);
     if (tune->vec > 0) p.sh.vec = tune->vec;
     if (tune->unroll > 0) p.sh.rw = tune->unroll;
     if (tune->bt > 0) p.sh.nrg = tune->bt;
@@ -203,7 +205,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     const size_t tile_rows = gated ? (bwd ? (size_t)(p.R + K - 1) + 2 * (size_t)p.R : 2 * (size_t)(p.R + K - 1))
                                    : (size_t)(p.R + K - 1) + (bwd ? p.R : 0);
     const size_t shmem = (size_t)p.sh.nbuf * tile_rows * cb_bytes;
-    if (shmem > kLdsBytesPerCU || cb_bytes % 1024) return -NPLM_DWCONV_ETUNING;
+    if (shmem > kLdsBytesPerCU || cb_bytes % 256) return -NPLM_DWCONV_ETUNING;
     if ((long long)(p.R + K) * row_bytes * (gated ? 2 : 1) + 2 * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
     p.ncb = ceil_div(row_bytes, cb_bytes);
     p.ntiles = ceil_div(T, p.R);

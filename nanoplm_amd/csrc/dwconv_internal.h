@@ -145,6 +145,36 @@ constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
     return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, (bf16 && K >= 9) ? 4 : 8, 2}
                : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
 }
+// Rows that are not a whole number of 2 KiB column blocks leave them partly empty. Two more column-block widths
+// cover the common cases, both with 4 bytes per lane (256-byte wave-columns) and K <= 9:
+//   768 bytes  (C = 768 and 1152 in bf16, the reference's default hidden and intermediate widths,
+//               modeling.py:42-43): 3 wave-columns, 3 row groups of 16 rows (48-row tiles, so that a tile in flight
+//               is still ~75 KiB per CU). Backward: 9 compute + 7 loader waves (3 at K = 9 in bf16, for the
+//               registers), two (dy, x) tile pairs (153 KiB). Forward: 9 compute + 4 loader waves, two x tiles of
+//               48 + K-1 rows (81 KiB at K = 7).
+//   1280 bytes (C = 640, 1280, 2560 in bf16), backward only: 5 wave-columns, 2 row groups of 12 rows (24-row
+//               tiles), 10 compute + 6 loader waves, 135 KiB.
+// Measured at T=131072, K=7, bf16 (us, 2 KiB blocks or sliding-window -> these): backward C=768 134 -> 125,
+// C=1152 205 -> 176, C=1536 252 -> 231, C=640 122 -> 108, C=1280 215 -> 195; forward C=1152 146 -> 113.
+// The forward otherwise keeps 2 KiB blocks, which it fills well enough from 3/4 up (1536-byte rows: 75 against
+// 80 us; 5120-byte rows at T=65536: 131 against 144 us in 1280-byte blocks).
+constexpr LdsShapeSel lds_narrow_shape(bool bwd, bool bf16, int K, int cb_bytes) {
+    if (cb_bytes == 768)
+        return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, (bf16 && K >= 9) ? 3 : 7, 2}
+                   : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, 4, 2};
+    return LdsShapeSel{bf16, bf16 ? 2 : 1, 12, 2, 5, 6, 2};      // 1280, backward
+}
+// 0 = the default column block, else 768 or 1280
+constexpr int lds_narrow_cb(bool bwd, int K, long long row_bytes) {
+    if (K > 9 || row_bytes % 2048 == 0) return 0;
+    if (bwd) return row_bytes % 768 == 0 ? 768 : (row_bytes % 1280 == 0 ? 1280 : 0);
+    const long long ncb2k = (row_bytes + 2047) / 2048;
+    return (row_bytes % 768 == 0 && ncb2k > 1 && row_bytes * 4 < ncb2k * 2048 * 3) ? 768 : 0;
+}
+constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_bytes) {
+    return lds_narrow_cb(bwd, K, row_bytes) ? lds_narrow_shape(bwd, bf16, K, lds_narrow_cb(bwd, K, row_bytes))
+                                            : lds_default_shape(bwd, bf16, K);
+}
 // Gated kernels (z = [u | g] input): 1 KiB column blocks, so that a u tile and a g tile fit where the plain
 // kernels hold one x tile: 4 wave-columns x 4 bytes per lane, 2 row groups, 4 loader waves. The gate
 // costs two transcendentals per element read, so the forward takes 32-row tiles (16 rows per wave: the

@@ -111,11 +111,11 @@ struct LdsShape {
     static constexpr int NROWS = R + K - 1;             // staged rows per tile
     static constexpr int CB_BYTES = NCW * 64 * VEC * E; // bytes of a row in one column block
     static constexpr int CB_CH = NCW * 64 * VEC;        // channels in one column block
-    static constexpr int NPIECE = CB_BYTES / 1024;      // 1 KiB direct loads per staged row
+    static constexpr int NPIECE = (CB_BYTES + 1023) / 1024;   // direct loads (1 KiB each, the last may be partial) per staged row
+    static constexpr bool WHOLE_PIECES = CB_BYTES % 1024 == 0;
     static constexpr int TILE_BYTES = NROWS * CB_BYTES;
     static constexpr int MAIL_BYTES = 2 * NRG * 16;     // forward: two sets of one 16-byte boundary record per row group
-    static_assert(CB_BYTES % 1024 == 0, "a column block must be a whole number of 1 KiB wave loads");
-    static_assert((NPIECE & (NPIECE - 1)) == 0, "pieces per row must be a power of two");
+    static_assert(CB_BYTES % 256 == 0, "a column block is a whole number of 256-byte wave-columns");
     static_assert(NROWS * CB_BYTES <= 65536, "ds_read immediate offsets are 16 bit");
 };
 
@@ -140,7 +140,9 @@ __device__ __forceinline__ void stage_rows(const void* __restrict__ src, char* d
 
 // Same as stage_rows, but every loader wave issues exactly CNT loads (surplus slots repeat the last
 // pair, lanes past the end of a narrow column block re-read its last 16 bytes), so that
-// "all but the newest CNT loads have landed" is a compile-time s_waitcnt.
+// "all but the newest CNT loads have landed" is a compile-time s_waitcnt. Column blocks that are not
+// a whole number of 1 KiB pieces mask the lanes past the end instead (their LDS slots belong to the
+// next row); a piece with no lane left is then skipped, which only the plain "wait for all" tolerates.
 template <typename SH, int CNT>
 __device__ __forceinline__ void stage_rows_fixed(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
                                                  size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw,
@@ -156,10 +158,11 @@ __device__ __forceinline__ void stage_rows_fixed(const void* __restrict__ src, c
         const int j = pair / SH::NPIECE;
         const int p = pair % SH::NPIECE;
         int boff = p * 1024 + lane * 16;
-        boff = boff < valid_bytes ? boff : valid_bytes - 16;
+        const bool inside = boff < valid_bytes;
+        boff = inside ? boff : valid_bytes - 16;
         const int so = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0;
         char* d = dst + j * SH::CB_BYTES + p * 1024;
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, boff, so, 0, 0);
+        if (SH::WHOLE_PIECES || inside) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, boff, so, 0, 0);
     }
 }
 
@@ -268,6 +271,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     constexpr int CNT = (SH::NROWS * SH::NPIECE + NWL - 1) / NWL;     // loads per loader wave per tile and tensor
     constexpr int BUF_BYTES = SH::TILE_BYTES * (GATED ? 2 : 1);
     static_assert(NBUF == 2 || NBUF == 3, "two or three tile buffers");
+    static_assert(NBUF == 2 || SH::WHOLE_PIECES, "three buffers count loads in flight: whole 1 KiB pieces only");
     static_assert(!GATED || NBUF == 2, "the gated forward is double-buffered");
     // Where LDS has 32 bytes to spare per row group, the loader waves (idle while their loads are in
     // flight) also run the boundary lookup for the next tile and leave the result in a mailbox behind

@@ -110,9 +110,11 @@ def test_kernel_sizes(K, dt):
     _check_case(*_random_case(LENS_MIX, 256, K, dt, dt, seed=K), f"K={K} {dt}")
 
 
-@pytest.mark.parametrize("C", [1, 7, 8, 24, 64, 72, 100, 128, 130, 520, 1000, 1024, 2048, 4104])
+@pytest.mark.parametrize("C", [1, 7, 8, 24, 64, 72, 100, 128, 130, 384, 520, 576, 640, 768, 1000, 1024, 1152, 1280, 2048,
+                               2560, 4104])
 def test_channel_counts(C):
-    """Every lane-slice width (8/4/2/1 channels per lane), partial wave-columns and odd channel counts."""
+    """Every lane-slice width (8/4/2/1 channels per lane), partial wave-columns, odd channel counts, and the row
+    widths that take 768- and 1280-byte column blocks in the LDS-staged kernels."""
     print(f"[case] C={C}", flush=True)
     _check_case(*_random_case([5, 1, 40, 2, 90, 3], C, 7, torch.bfloat16, torch.bfloat16, seed=C), f"C={C}")
     _check_case(*_random_case([5, 1, 40, 2, 90, 3], C, 3, torch.float32, torch.float32, seed=C), f"C={C} fp32")
@@ -337,7 +339,8 @@ def test_rows_beyond_2_and_4_gib_offsets():
 
 
 @pytest.mark.parametrize("K,C,dt", [(7, 1024, torch.bfloat16), (7, 512, torch.float32), (31, 1024, torch.bfloat16),
-                                    (9, 1024, torch.bfloat16)])
+                                    (9, 1024, torch.bfloat16), (7, 768, torch.bfloat16), (9, 1152, torch.bfloat16),
+                                    (9, 1280, torch.bfloat16), (5, 576, torch.float32), (3, 320, torch.float32)])
 @pytest.mark.parametrize("seq_len,nbt", [(64, 0), (96, 24), (17, 10), (512, 7)])
 def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
     """Equal-length sequences put boundaries at a fixed period of tiles; the LDS kernels rotate the tile slots
