@@ -192,7 +192,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    p.sh = gated ? lds_gated_shape(bwd, bf16) : lds_shape_for(bwd, bf16, K, (long long)C * E);
+    p.sh = gated ? lds_gated_shape(bwd, bf16, lds_gated_narrow((long long)C * E), K) : lds_shape_for(bwd, bf16, K, (long long)C * E);
     if (tune->vec > 0) p.sh.vec = tune->vec;
     if (tune->unroll > 0) p.sh.rw = tune->unroll;
     if (tune->bt > 0) p.sh.nrg = tune->bt;
@@ -502,14 +502,15 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     rc = make_lds_plan(false, bf16, T, C, K, nullptr, &lp, true);
     if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
     const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
+    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4));
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.ncb * lp.nbt);
     hipStream_t s = (hipStream_t)stream;
     switch (K) {
-        case 3: return (int)launch_fwd_lds_gated_k3(bf16, la, g, grid, s);
-        case 5: return (int)launch_fwd_lds_gated_k5(bf16, la, g, grid, s);
-        case 7: return (int)launch_fwd_lds_gated_k7(bf16, la, g, grid, s);
-        case 9: return (int)launch_fwd_lds_gated_k9(bf16, la, g, grid, s);
+        case 3: return (int)launch_fwd_lds_gated_k3(bf16, narrow, la, g, grid, s);
+        case 5: return (int)launch_fwd_lds_gated_k5(bf16, narrow, la, g, grid, s);
+        case 7: return (int)launch_fwd_lds_gated_k7(bf16, narrow, la, g, grid, s);
+        case 9: return (int)launch_fwd_lds_gated_k9(bf16, narrow, la, g, grid, s);
     }
     return -NPLM_DWCONV_EUNSUPPORTED;
 }
@@ -550,14 +551,15 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         return -NPLM_DWCONV_EWORKSPACE;
     float* part = reinterpret_cast<float*>(workspace);
     const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
+    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4));
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.ncb * lp.nbt);
     hipError_t e = hipErrorInvalidConfiguration;
     switch (K) {
-        case 3: e = launch_bwd_lds_gated_k3(bf16, la, g, grid, s); break;
-        case 5: e = launch_bwd_lds_gated_k5(bf16, la, g, grid, s); break;
-        case 7: e = launch_bwd_lds_gated_k7(bf16, la, g, grid, s); break;
-        case 9: e = launch_bwd_lds_gated_k9(bf16, la, g, grid, s); break;
+        case 3: e = launch_bwd_lds_gated_k3(bf16, narrow, la, g, grid, s); break;
+        case 5: e = launch_bwd_lds_gated_k5(bf16, narrow, la, g, grid, s); break;
+        case 7: e = launch_bwd_lds_gated_k7(bf16, narrow, la, g, grid, s); break;
+        case 9: e = launch_bwd_lds_gated_k9(bf16, narrow, la, g, grid, s); break;
     }
     if (e != hipSuccess) return (int)e;
     const long long n_out = (long long)(K + 1) * C;

@@ -94,8 +94,10 @@ struct LdsShapeSel {
     hipError_t launch_bwd_lds_k##KK(const LdsShapeSel& sh, bool wdx, bool wdw, const ConvPtrs& p,         \
                                     const LdsGeo& g, dim3 grid, hipStream_t s);
 #define NPLM_DECLARE_LDS_GATED_K(KK)                                                                      \
-    hipError_t launch_fwd_lds_gated_k##KK(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s); \
-    hipError_t launch_bwd_lds_gated_k##KK(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+    hipError_t launch_fwd_lds_gated_k##KK(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, \
+                                          hipStream_t s);                                                 \
+    hipError_t launch_bwd_lds_gated_k##KK(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, \
+                                          hipStream_t s);
 NPLM_DECLARE_LDS_GATED_K(3)
 NPLM_DECLARE_LDS_GATED_K(5)
 NPLM_DECLARE_LDS_GATED_K(7)
@@ -180,7 +182,14 @@ constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_by
 // costs two transcendentals per element read, so the forward takes 32-row tiles (16 rows per wave: the
 // K-1 halo rows it re-gates weigh less; 2 x 2 x 38 KiB = 152 KiB of LDS at K = 7), the backward 16-row
 // tiles (2 x (22 + 16 + 16) KiB = 108 KiB).
-constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16) {
+// Rows that are a multiple of 768 bytes but not of 1 KiB (C = 1152 in bf16, the reference's default
+// intermediate width) take 768-byte column blocks: 3 wave-columns; forward 2 row groups of 16 rows, backward
+// 3 row groups of 8 rows with 3 loader waves (12 waves: the registers of the gated backward need it; at K = 9 in
+// bf16 2 row groups and 2 loader waves, 8 waves).
+constexpr bool lds_gated_narrow(long long row_bytes) { return row_bytes % 768 == 0 && row_bytes % 1024 != 0; }
+constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16, bool narrow = false, int K = 7) {
+    if (narrow && bwd && bf16 && K >= 9) return LdsShapeSel{true, 2, 8, 2, 3, 2, 2};
+    if (narrow) return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 3, 3, 3, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 3, 4, 2};
     return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, 2, 4, 4, 2};
 }
 constexpr bool lds_gated_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }

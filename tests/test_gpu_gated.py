@@ -39,7 +39,8 @@ def _check(z, cu, w, b, dy, what, residual=False):
 
 
 @pytest.mark.parametrize("K", [3, 5, 7, 9])
-@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.bfloat16, 520), (torch.float32, 256), (torch.float32, 768)])
+@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.bfloat16, 520), (torch.float32, 256), (torch.float32, 768),
+                                   (torch.bfloat16, 1152), (torch.float32, 576)])
 def test_gated_kernel_sizes_and_widths(K, dt, C):
     print(f"[case] gated K={K} C={C} {dt}", flush=True)
     _check(*_case(LENS_MIX, C, K, dt, dt, seed=K + C), f"gated K={K} C={C} {dt}")
