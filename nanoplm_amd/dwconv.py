@@ -32,6 +32,28 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+class _launch_on:
+    """Context for one library call: makes the tensor's device current (nothing to do when it already is, the
+    usual case) and holds the raw handle of that device's current stream in ``.stream``."""
+    __slots__ = ("idx", "prev", "stream")
+
+    def __init__(self, t: torch.Tensor):
+        self.prev = torch.cuda.current_device()
+        self.idx = self.prev if t.device.index is None else t.device.index
+        self.stream = None
+
+    def __enter__(self):
+        if self.idx != self.prev:
+            torch.cuda.set_device(self.idx)
+        self.stream = torch._C._cuda_getCurrentRawStream(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.idx != self.prev:
+            torch.cuda.set_device(self.prev)
+        return False
+
+
 def _validate(x, cu_seqlens, weight, bias):
     """Shape/dtype/device checks shared by forward and backward. Returns (T, C, K, S)."""
     if not isinstance(x, torch.Tensor) or x.dim() != 2:
@@ -76,8 +98,8 @@ def varlen_dwconv_fwd(x, cu_seqlens, weight, bias=None, *, residual: bool = Fals
     if bias is not None:
         bias = bias.to(weight.dtype).contiguous()
     y = torch.empty_like(x)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _launch_on(x) as dev:
+        stream = dev.stream
         flags = _lib.RESIDUAL if residual else 0
         args = (_ptr(x), _ptr(cu_seqlens), _ptr(weight), _ptr(bias), _ptr(y), T, C, K, S,
                 _DTYPES[x.dtype], _DTYPES[weight.dtype])
@@ -111,14 +133,14 @@ def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, 
     dx = torch.empty_like(x) if need_dx else None
     dw = torch.empty((C, K), dtype=torch.float32, device=x.device) if need_dw else None
     db = torch.empty((C,), dtype=torch.float32, device=x.device) if need_dw else None
-    with torch.cuda.device(x.device):
+    with _launch_on(x) as dev:
         if need_dw and workspace is None:
             if tuning is None:
                 nbytes = int(lib.nplm_dwconv_bwd_workspace_bytes(T, C, K, act))
             else:
                 nbytes = int(lib.nplm_dwconv_bwd_slabs(T, C, K, act, tuning)) * (K + 1) * C * 4
             workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
-        stream = torch.cuda.current_stream().cuda_stream
+        stream = dev.stream
         flags = _lib.RESIDUAL if residual else 0
         args = (_ptr(x), _ptr(dy), _ptr(cu_seqlens), _ptr(weight), _ptr(dx), _ptr(dw), _ptr(db),
                 _ptr(workspace), 0 if workspace is None else workspace.numel() * workspace.element_size(),
@@ -136,9 +158,8 @@ def check_cu_seqlens(cu_seqlens: torch.Tensor, T: int) -> None:
     if not cu_seqlens.is_cuda or cu_seqlens.dtype != torch.int32:
         raise TypeError("cu_seqlens must be an int32 tensor on a ROCm device")
     lib = _lib.load()
-    with torch.cuda.device(cu_seqlens.device):
-        rc = lib.nplm_dwconv_check_cu(_ptr(cu_seqlens.contiguous()), cu_seqlens.numel() - 1, T,
-                                      torch.cuda.current_stream().cuda_stream)
+    with _launch_on(cu_seqlens) as dev:
+        rc = lib.nplm_dwconv_check_cu(_ptr(cu_seqlens.contiguous()), cu_seqlens.numel() - 1, T, dev.stream)
     _lib.check(rc, "nplm_dwconv_check_cu")
 
 

@@ -22,7 +22,7 @@ import torch
 import torch.nn.functional as F
 
 from . import _lib
-from .dwconv import _DTYPES, _ptr, varlen_dwconv
+from .dwconv import _DTYPES, _launch_on, _ptr, varlen_dwconv
 
 
 def gated_supported(z: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -59,10 +59,10 @@ def gated_dwconv_fwd(z, cu_seqlens, weight, bias=None, *, residual: bool = False
     if bias is not None:
         bias = bias.to(weight.dtype).contiguous()
     y = torch.empty((T, C), dtype=z.dtype, device=z.device)
-    with torch.cuda.device(z.device):
+    with _launch_on(z) as dev:
         rc = lib.nplm_dwconv_gated_fwd(_ptr(z), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(bias), _ptr(y), T, C, K, S,
                                        _DTYPES[z.dtype], _DTYPES[weight.dtype], _lib.RESIDUAL if residual else 0,
-                                       torch.cuda.current_stream().cuda_stream)
+                                       dev.stream)
     _lib.check(rc, "nplm_dwconv_gated_fwd")
     return y
 
@@ -80,12 +80,12 @@ def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
     dz = torch.empty_like(z)
     dw = torch.empty((C, K), dtype=torch.float32, device=z.device)
     db = torch.empty((C,), dtype=torch.float32, device=z.device)
-    with torch.cuda.device(z.device):
+    with _launch_on(z) as dev:
         nbytes = int(lib.nplm_dwconv_gated_bwd_workspace_bytes(T, C, K, act))
         ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=z.device)
         rc = lib.nplm_dwconv_gated_bwd(_ptr(z), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(dz), _ptr(dw),
                                        _ptr(db), _ptr(ws), ws.numel(), T, C, K, S, act, _DTYPES[weight.dtype],
-                                       _lib.RESIDUAL if residual else 0, torch.cuda.current_stream().cuda_stream)
+                                       _lib.RESIDUAL if residual else 0, dev.stream)
     _lib.check(rc, "nplm_dwconv_gated_bwd")
     return dz, dw, db
 
