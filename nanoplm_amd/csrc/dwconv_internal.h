@@ -181,16 +181,17 @@ constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_by
 // kernels hold one x tile: 4 wave-columns x 4 bytes per lane, 2 row groups, 4 loader waves. The gate
 // costs two transcendentals per element read, so the forward takes 32-row tiles (16 rows per wave: the
 // K-1 halo rows it re-gates weigh less; 2 x 2 x 38 KiB = 152 KiB of LDS at K = 7), the backward 16-row
-// tiles (2 x (22 + 16 + 16) KiB = 108 KiB).
+// tiles (2 x (22 + 16 + 16) KiB = 108 KiB). Taller backward tiles would stream better (K = 3, whose registers
+// allow a third row group: 297 -> 254 us at T=131072, C=1024) but spill from K = 5 on (K = 7: 295 -> 328 us).
 // Rows that are a multiple of 768 bytes but not of 1 KiB (C = 1152 in bf16, the reference's default
 // intermediate width) take 768-byte column blocks: 3 wave-columns; forward 2 row groups of 16 rows, backward
 // 3 row groups of 8 rows with 3 loader waves (12 waves: the registers of the gated backward need it).
 constexpr bool lds_gated_narrow(long long row_bytes) { return row_bytes % 768 == 0 && row_bytes % 1024 != 0; }
 constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16, bool narrow = false, int K = 7) {
-    (void)K;   // one shape for every K <= 9 (at K = 9 in bf16 the backward spills 5 registers; a variant with fewer
-               // waves and no spill measured slower: 440 against 334 us at T=131072, C=1152)
+    // narrow: one shape for every K <= 9 (at K = 9 in bf16 the backward spills 5 registers; a variant with fewer
+    // waves and no spill measured slower: 440 against 334 us at T=131072, C=1152)
     if (narrow) return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 3, 3, 3, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 3, 4, 2};
-    return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, 2, 4, 4, 2};
+    return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, (bwd && K == 3) ? 3 : 2, 4, 4, 2};
 }
 constexpr bool lds_gated_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
 constexpr int default_maxt(bool bwd, int K, int vec) {
