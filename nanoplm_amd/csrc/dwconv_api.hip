@@ -1,5 +1,6 @@
 // C ABI of libnplm_dwconv (see include/nplm_dwconv.h): argument checks, launch planning and
-// dispatch to the per-K launchers. Host code only; the kernels live in dwconv_kernels.h.
+// dispatch to the per-K launchers. Host code only; the kernels live in dwconv_kernels.h and
+// dwconv_lds_kernels.h.
 //
 // The entry points stand where a conv module's forward/backward would sit on the reference's
 // packed path (src/nanoplm/pretraining/models/modern_bert/modeling.py:421-439; backward driven by
@@ -167,13 +168,12 @@ bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     return (long long)C * E >= 1024;
 }
 
-// Whether they are also the faster choice. A block owns one column block (2 KiB, 768 bytes for rows that
-// are a multiple of that, 1 KiB at K = 31) of its rows and the grid's time follows the number of column
-// blocks, so a row that fills its column blocks poorly wastes lanes and loader slots. Measured on MI355X
-// (T=131072, K=7, bf16 rows of 1024 .. 10240 bytes and fp32 rows of 1024 .. 8192 bytes): LDS-staged wins
-// for a single column block filled to 5/8 or more; for several, the backward needs them filled to 4/5
-// on average (rows of 2560 bytes: 260 against 215 us), the forward only to 11/20 (same rows: 143 against
-// 154 us); the sliding-window kernels win otherwise (e.g. rows of 1024 bytes).
+// Whether they are also the faster choice. A block owns one column block of its rows (1 KiB by default,
+// see lds_shape_for) and the grid's time follows the number of column blocks, so a row that fills its
+// column blocks poorly wastes lanes and loader slots. Measured on MI355X (T=131072, K=7, bf16 rows of
+// 1024 .. 10240 bytes and fp32 rows of 1024 .. 8192 bytes): LDS-staged wins for a single column block
+// filled to 5/8 or more; for several, the backward needs them filled to 4/5 on average, the forward only
+// to 11/20; the sliding-window kernels win otherwise.
 bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     if (!lds_eligible(bf16, T, C, K, align_bits)) return false;
     if (K > 9 && bwd) return false;        // K = 31: only the forward fits its registers

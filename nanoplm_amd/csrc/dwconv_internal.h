@@ -133,45 +133,45 @@ constexpr int default_unroll(bool bwd, int K, int vec) {
 }
 // Kernel sizes the LDS-staged kernels are built for.
 constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 31; }
-// Default shapes (a block always owns 2 KiB of every row of its tile, 16-row tiles):
-//   forward : 4 wave-columns x 8 bytes per lane, 2 row groups of 8 rows, 4 loader waves; two x tiles
-//             of 16 + K-1 rows (88 KiB of LDS at K = 7).
-//   backward: 8 wave-columns x 4 bytes per lane, 1 row group of 16 rows, 8 loader waves; two
-//             (dy tile of 16 + K-1 rows, x tile of 16 rows) pairs = 152 KiB of the 160 KiB a CU has
-//             (exactly 160 KiB at K = 9). Four bytes per lane keep the 16-row register tile
-//             (dx accumulators + x rows + weights + dw/db) under the 128 registers 16 waves leave.
+// Default shapes: a block owns 1 KiB of every row of a 32-row tile.
+//   forward : 2 wave-columns x 8 bytes per lane, 4 row groups of 8 rows, 4 loader waves; two x tiles of
+//             32 + K-1 rows (76 KiB of LDS at K = 7).
+//   backward: 4 wave-columns x 4 bytes per lane, 2 row groups of 16 rows, 3 loader waves; two
+//             (dy tile of 32 + K-1 rows, x tile of 32 rows) pairs = 140 KiB of the 160 KiB a CU has.
+//             Four bytes per lane keep the 16-row register tile (dx accumulators + x rows + weights + dw/db)
+//             in the registers 11 waves leave (168; K = 9 in bf16 needs more than 128).
+// Measured at T=131072, C=1024, K=7, bf16 against 16-row tiles on 2 KiB column blocks (the same bytes per
+// tile, more halo rows per output row, twice the barriers): forward 98 -> 95 us, backward + finalize
+// 155 -> 151 us; more loader waves than these are slower (backward with 4: 153, with 5: 155 us).
 constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
-    if (K >= 15)   // long kernels: 1 KiB column blocks and 32-row tiles, so that tile + K-1 halo rows still fit twice
+    if (K >= 15)   // long kernels: 32-row tiles of 16-row waves, so that tile + K-1 halo rows still fit twice
         return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 2, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
-    // (K = 9 in bf16 needs more than 128 registers: 4 loader waves there, which leaves 168)
-    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 1, 8, (bf16 && K >= 9) ? 4 : 8, 2}
-               : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};
+    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 3, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 4, 2, 4, 2};
 }
-// Rows that are not a whole number of 2 KiB column blocks leave them partly empty. Two more column-block widths
-// cover the common cases, both with 4 bytes per lane (256-byte wave-columns) and K <= 9:
-//   768 bytes  (C = 768 and 1152 in bf16, the reference's default hidden and intermediate widths,
-//               modeling.py:42-43): 3 wave-columns, 3 row groups of 16 rows (48-row tiles, so that a tile in flight
-//               is still ~75 KiB per CU). Backward: 9 compute + 7 loader waves (3 at K = 9 in bf16, for the
-//               registers), two (dy, x) tile pairs (153 KiB). Forward: 9 compute + 4 loader waves, two x tiles of
-//               48 + K-1 rows (81 KiB at K = 7).
-//   1280 bytes (C = 640, 1280, 2560 in bf16), backward only: 5 wave-columns, 2 row groups of 12 rows (24-row
-//               tiles), 10 compute + 6 loader waves, 135 KiB.
-// Measured at T=131072, K=7, bf16 (us, 2 KiB blocks or sliding-window -> these): backward C=768 134 -> 125,
-// C=1152 205 -> 176, C=1536 252 -> 231, C=640 122 -> 108, C=1280 215 -> 195; forward C=1152 146 -> 113.
-// The forward otherwise keeps 2 KiB blocks, which it fills well enough from 3/4 up (1536-byte rows: 75 against
-// 80 us; 5120-byte rows at T=65536: 131 against 144 us in 1280-byte blocks).
+constexpr int kLdsDefaultCb = 1024;
+// Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block
+// widths cover the common cases (K <= 9):
+//   backward, 768 bytes (C = 768 and 1152 in bf16, the reference's default hidden and intermediate widths,
+//       modeling.py:42-43): 3 wave-columns x 4 bytes per lane, 3 row groups of 16 rows (48-row tiles, so that a
+//       tile in flight is still ~75 KiB per CU); 9 compute + 7 loader waves (3 at K = 9 in bf16, for the
+//       registers), two (dy, x) tile pairs (153 KiB).
+//   backward, 1280 bytes (C = 640, 1280 in bf16): 5 wave-columns x 4 bytes per lane, 2 row groups of 12 rows,
+//       10 compute + 6 loader waves, 135 KiB.
+//   forward, 2 KiB for rows between 1280 and 2047 bytes (C = 640 .. 1023 in bf16), which fill one such block
+//       better than two of 1 KiB: 4 wave-columns x 8 bytes per lane, 2 row groups of 8 rows, 4 loader waves.
+// Measured at T=131072, K=7, bf16 (us, default blocks -> these): backward C=768 140 -> 124, C=1152 200 -> 175,
+// C=640 135 -> 106, C=1280 208 -> 193; forward C=768 83 -> 76. The forward gains nothing from 768-byte blocks
+// (C=1152: 113 against 115, C=2304 at T=65536: 119 against 110).
 constexpr LdsShapeSel lds_narrow_shape(bool bwd, bool bf16, int K, int cb_bytes) {
-    if (cb_bytes == 768)
-        return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, (bf16 && K >= 9) ? 3 : 7, 2}
-                   : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, 4, 2};
-    return LdsShapeSel{bf16, bf16 ? 2 : 1, 12, 2, 5, 6, 2};      // 1280, backward
+    if (!bwd) return LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};          // 2048, forward
+    if (cb_bytes == 768) return LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, (bf16 && K >= 9) ? 3 : 7, 2};
+    return LdsShapeSel{bf16, bf16 ? 2 : 1, 12, 2, 5, 6, 2};                  // 1280, backward
 }
-// 0 = the default column block, else 768 or 1280
+// 0 = the default column block, else 768 or 1280 (backward), 2048 (forward)
 constexpr int lds_narrow_cb(bool bwd, int K, long long row_bytes) {
-    if (K > 9 || row_bytes % 2048 == 0) return 0;
-    if (bwd) return row_bytes % 768 == 0 ? 768 : (row_bytes % 1280 == 0 ? 1280 : 0);
-    const long long ncb2k = (row_bytes + 2047) / 2048;
-    return (row_bytes % 768 == 0 && ncb2k > 1 && row_bytes * 4 < ncb2k * 2048 * 3) ? 768 : 0;
+    if (K > 9 || row_bytes % kLdsDefaultCb == 0) return 0;
+    if (!bwd) return (row_bytes >= 1280 && row_bytes < 2048) ? 2048 : 0;
+    return row_bytes % 768 == 0 ? 768 : (row_bytes % 1280 == 0 ? 1280 : 0);
 }
 constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_bytes) {
     return lds_narrow_cb(bwd, K, row_bytes) ? lds_narrow_shape(bwd, bf16, K, lds_narrow_cb(bwd, K, row_bytes))
