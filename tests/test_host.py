@@ -71,6 +71,17 @@ def test_workspace_bytes_arithmetic():
     assert lib.nplm_dwconv_bwd_workspace_bytes(100, 64, 4, 1) == 0
 
 
+def test_column_block_width_follows_the_row_width():
+    """The LDS-staged backward deals one token block per CU and column block, so its slab count (256 / column
+    blocks per row) shows which column-block width the planner picked: 1 KiB by default, 768 bytes for rows that
+    are a multiple of that (C = 768, 1152 in bf16; 576 in fp32), 1280 bytes for rows of 1280 and 2560 bytes."""
+    lib = _lib.load()
+    lds = _lib.Tuning(algo=2)
+    for (C, act, slabs) in [(1024, 1, 128), (2048, 1, 64), (512, 1, 256), (896, 1, 128), (768, 1, 128),
+                            (1152, 1, 85), (640, 1, 256), (1280, 1, 128), (576, 0, 85), (512, 0, 128)]:
+        assert lib.nplm_dwconv_bwd_slabs(131072, C, 7, act, lds) == slabs, (C, act)
+
+
 # ---- boundary cursor ---------------------------------------------------------------------------
 def _intervals(cu, T, start=0, step=1, relocate_every=0):
     cu = np.ascontiguousarray(np.asarray(cu, dtype=np.int32))
