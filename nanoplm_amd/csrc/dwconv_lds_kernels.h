@@ -2,7 +2,7 @@
 // for K <= 9, the forward also for K = 31.
 //
 // A block owns tiles of R = RW*NRG consecutive token rows x one column block of NCW*64*VEC channels
-// (2 KiB of every row at the default sizes). Its waves have two roles:
+// (1 KiB of every row of a 32-row tile at the default sizes). Its waves have two roles:
 //
 //   loader waves (NWL)   issue direct global->LDS loads (buffer_load ... lds, 16 B per lane,
 //                        consecutive lanes consecutive addresses) for the NEXT tile and its K-1 halo
