@@ -32,6 +32,9 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # fast path; public API otherwise
+
+
 class _launch_on:
     """Context for one library call: makes the tensor's device current (nothing to do when it already is, the
     usual case) and holds the raw handle of that device's current stream in ``.stream``."""
@@ -45,7 +48,8 @@ class _launch_on:
     def __enter__(self):
         if self.idx != self.prev:
             torch.cuda.set_device(self.idx)
-        self.stream = torch._C._cuda_getCurrentRawStream(self.idx)
+        self.stream = (_raw_stream(self.idx) if _raw_stream is not None
+                       else torch.cuda.current_stream(self.idx).cuda_stream)
         return self
 
     def __exit__(self, *exc):
