@@ -176,7 +176,7 @@ bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
 // to 11/20; the sliding-window kernels win otherwise.
 bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     if (!lds_eligible(bf16, T, C, K, align_bits)) return false;
-    if (K > 9 && bwd) return false;        // K = 31: only the forward fits its registers
+    if (K > 9 && bwd) return false;        // K = 15, 31: only the forward is built (the fused backward does not fit its registers)
     const long long E = bf16 ? 2 : 4;
     const long long row_bytes = (long long)C * E;
     const LdsShapeSel sh = lds_shape_for(bwd, bf16, K, row_bytes);
@@ -245,6 +245,7 @@ hipError_t launch_fwd_lds(int K, const LdsPlan& p, const ConvPtrs& a, const LdsG
         case 5: return launch_fwd_lds_k5(p.sh, a, g, grid, s);
         case 7: return launch_fwd_lds_k7(p.sh, a, g, grid, s);
         case 9: return launch_fwd_lds_k9(p.sh, a, g, grid, s);
+        case 15: return launch_fwd_lds_k15(p.sh, a, g, grid, s);
         case 31: return launch_fwd_lds_k31(p.sh, a, g, grid, s);
     }
     return hipErrorInvalidConfiguration;
@@ -257,6 +258,7 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
         case 5: return launch_bwd_lds_k5(p.sh, wdx, wdw, a, g, grid, s);
         case 7: return launch_bwd_lds_k7(p.sh, wdx, wdw, a, g, grid, s);
         case 9: return launch_bwd_lds_k9(p.sh, wdx, wdw, a, g, grid, s);
+        case 15: return launch_bwd_lds_k15(p.sh, wdx, wdw, a, g, grid, s);
         case 31: return launch_bwd_lds_k31(p.sh, wdx, wdw, a, g, grid, s);
     }
     return hipErrorInvalidConfiguration;

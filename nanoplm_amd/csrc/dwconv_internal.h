@@ -107,6 +107,7 @@ NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
 NPLM_DECLARE_LDS_K(7)
 NPLM_DECLARE_LDS_K(9)
+NPLM_DECLARE_LDS_K(15)
 NPLM_DECLARE_LDS_K(31)
 #undef NPLM_DECLARE_LDS_K
 NPLM_DECLARE_K(3)
@@ -132,7 +133,7 @@ constexpr int default_unroll(bool bwd, int K, int vec) {
     return vec >= 8 ? 4 : 8;
 }
 // Kernel sizes the LDS-staged kernels are built for.
-constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 31; }
+constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 15 || K == 31; }
 // Default shapes: a block owns 1 KiB of every row of a 32-row tile.
 //   forward : 2 wave-columns x 8 bytes per lane, 4 row groups of 8 rows, 4 loader waves; two x tiles of
 //             32 + K-1 rows (76 KiB of LDS at K = 7).

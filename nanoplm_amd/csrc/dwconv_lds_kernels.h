@@ -1,5 +1,5 @@
 // LDS-staged, software-pipelined kernels of the varlen depthwise conv (gfx950, wave64): both passes
-// for K <= 9, the forward also for K = 31.
+// for K <= 9, the forward also for K = 15 and 31.
 //
 // A block owns tiles of R = RW*NRG consecutive token rows x one column block of NCW*64*VEC channels
 // (1 KiB of every row of a 32-row tile at the default sizes). Its waves have two roles:

@@ -340,7 +340,8 @@ def test_rows_beyond_2_and_4_gib_offsets():
 
 @pytest.mark.parametrize("K,C,dt", [(7, 1024, torch.bfloat16), (7, 512, torch.float32), (31, 1024, torch.bfloat16),
                                     (9, 1024, torch.bfloat16), (7, 768, torch.bfloat16), (9, 1152, torch.bfloat16),
-                                    (9, 1280, torch.bfloat16), (5, 576, torch.float32), (3, 320, torch.float32)])
+                                    (9, 1280, torch.bfloat16), (5, 576, torch.float32), (3, 320, torch.float32),
+                                    (15, 1024, torch.bfloat16)])
 @pytest.mark.parametrize("seq_len,nbt", [(64, 0), (96, 24), (17, 10), (512, 7)])
 def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
     """Equal-length sequences put boundaries at a fixed period of tiles; the LDS kernels rotate the tile slots
@@ -358,8 +359,8 @@ def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
         y = npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=tf)
         try:
             dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=tf)
-        except RuntimeError:         # no LDS-staged backward at K = 31
-            assert algo == 2 and K == 31
+        except RuntimeError:         # no LDS-staged backward at K = 15, 31
+            assert algo == 2 and K in (15, 31)
             dx = None
         outs.append((y, dx))
     assert torch.equal(outs[0][0], outs[1][0])
