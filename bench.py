@@ -9,10 +9,17 @@ configuration 3 of nanoplm_amd.workloads (T=131072 packed tokens, C=1024, K=7, b
 headline metric is quoted on. Three input/output sets (> 256 MB each) are rotated so no step reads
 a tensor that is still in the Infinity Cache.
 
+Order of one run: an untimed pre-warm (the same forward + backward launches for --prewarm-ms, so that
+the GPU has reached its steady clocks and every buffer has been touched before anything is timed),
+W warm-up steps, then the loop of K steps timed --reps times in a row, each repetition bracketed by
+a stream synchronisation on both sides.
+
 One JSON line is printed:
-  value         tokens/s over the K timed steps (wall clock, stream synchronised on both sides)
+  value         tokens/s of the median repetition of the K timed steps (wall clock); ms_per_step_min
+                and ms_per_step_reps give the fastest repetition and all of them
   roofline      the dominant kernel (the fused backward): algorithmic bytes per launch divided by its
-                average duration, measured with HIP events recorded on the launch stream
+                median duration over at least 50 launches, measured with HIP events recorded on the
+                launch stream (median_us, min_us and the mean avg_us are all printed)
   roofline_fwd  the same for the forward kernel (informational)
   back_to_back_us  span of 30 consecutive launches of one pass divided by 30 (informational: an event
                 record ends a kernel with a cache write-back that consecutive launches overlap)
@@ -36,11 +43,13 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and
 # scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
-# profiles/): keyed by (workload name, kernel).
+# profiles/bench_cfg3_hbm_traffic.md): keyed by (workload name, kernel). Counters cannot be read from
+# inside this process, so a workload without an entry reports traffic = null and says why.
 MEASURED_TRAFFIC = {
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 545113439,    # 1.015 x algorithmic
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 824575990,   # 1.024 x algorithmic
 }
+MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
 
 def _hip():
@@ -128,6 +137,9 @@ def main():
     ap.add_argument("--gated", action="store_true",
                     help="gated variant: input z = [x_proj | gate] of width 2C, conv over x_proj * silu(gate) "
                          "(informational; per-kernel figures then bracket backward + finalize together)")
+    ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
+    ap.add_argument("--prewarm-ms", type=float, default=1000.0,
+                    help="untimed steps run for this long before the warm-up steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=65536)
     args = ap.parse_args()
@@ -195,16 +207,29 @@ def main():
         if fwd_bwd:
             bwd(i)
 
-    # ---- whole-step throughput -----------------------------------------------------------------
-    for i in range(args.warmup):
-        step(i)
+    # ---- untimed pre-warm: the same launches until the clocks have settled --------------------------
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    prewarm_steps = 0
+    while (time.perf_counter() - t0) * 1e3 < args.prewarm_ms:
+        for i in range(50):
+            step(prewarm_steps + i)
+        prewarm_steps += 50
+        torch.cuda.synchronize()
+    prewarm_ms = (time.perf_counter() - t0) * 1e3
+
+    # ---- whole-step throughput: W warm-up steps, then K timed steps, repeated ------------------------
+    for i in range(args.warmup):
         step(i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    rep_ms = []
+    for _ in range(max(1, args.reps)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(i)
+        torch.cuda.synchronize()
+        rep_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
+    ms_per_step = statistics.median(rep_ms)
     tokens_per_s = T / (ms_per_step / 1e3)
 
     # ---- per-kernel durations with HIP events on the launch stream ---------------------------------
@@ -212,7 +237,7 @@ def main():
     # synchronisation, with one pair of events per step around the kernel being measured; one pass
     # over the steps per kernel, so that a step never carries more than two event records (every
     # record ends the kernel before it with a cache write-back, which the kernel after it pays for).
-    n_ev = min(max(args.steps, 10), 100)
+    n_ev = min(max(args.steps, MIN_EVENT_LAUNCHES), 100)
     evs = [HipEvents(4) for _ in range(n_ev)]
 
     def event_pass(which):
@@ -247,7 +272,6 @@ def main():
         event_pass("fin")
         fin_us = [e.elapsed_us(2, 3) for e in evs]
     ev = evs[0]
-    fwd_avg = statistics.fmean(fwd_us)
     fwd_bytes = wl.algorithmic_bytes("fwd")
     bwd_bytes = wl.algorithmic_bytes("bwd") if fwd_bwd else 0
     if args.gated:       # z is read once more per pass and dz is twice as wide as dx
@@ -256,18 +280,26 @@ def main():
         bwd_bytes += 2 * tce
     step_bytes = fwd_bytes + bwd_bytes
 
-    def roof(nbytes, us, kernel):
-        gbps = nbytes / us / 1e3
-        return {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
-                "traffic": None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel)), "kernel": kernel, "avg_us": us,
-                "algorithmic_bytes": nbytes}
+    def roof(nbytes, samples_us, kernel):
+        med = statistics.median(samples_us)
+        gbps = nbytes / med / 1e3
+        traffic = None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel))
+        r = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+             "traffic": traffic, "kernel": kernel, "median_us": med, "min_us": min(samples_us),
+             "avg_us": statistics.fmean(samples_us), "launches": len(samples_us), "algorithmic_bytes": nbytes}
+        if traffic is None:
+            r["traffic_note"] = ("no rocprofv3 FETCH_SIZE/WRITE_SIZE measurement is kept for this workload/variant; "
+                                 "the counters are read by the profiler, not by this process")
+        return r
 
     out = {
         "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
                   if args.config == 3 and not args.gated else
                   f"varlen {'gated ' if args.gated else ''}dwconv {wl.passes} tokens/s ({wl.name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "ms_per_step_min": min(rep_ms), "reps": len(rep_ms),
+        "ms_per_step_reps": [round(v, 5) for v in rep_ms], "prewarm_ms": prewarm_ms, "prewarm_steps": prewarm_steps,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
         "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
@@ -277,11 +309,11 @@ def main():
         "step_frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
     }
     if fwd_bwd:
-        out["roofline"] = roof(bwd_bytes, statistics.fmean(bwd_us), "backward")
-        out["roofline_fwd"] = roof(fwd_bytes, fwd_avg, "forward")
-        out["finalize_avg_us"] = statistics.fmean(fin_us)
+        out["roofline"] = roof(bwd_bytes, bwd_us, "backward")
+        out["roofline_fwd"] = roof(fwd_bytes, fwd_us, "forward")
+        out["finalize_median_us"] = statistics.median(fin_us)
     else:
-        out["roofline"] = roof(fwd_bytes, fwd_avg, "forward")
+        out["roofline"] = roof(fwd_bytes, fwd_us, "forward")
 
     # ---- the same launches back to back (no event between them): each figure is the span of N launches
     # divided by N, so it holds a launch gap but no end-of-kernel cache write-back forced by an event --
