@@ -199,7 +199,11 @@ class VarlenDWConv1dFunction(torch.autograd.Function):
 
 
 def varlen_dwconv(x, cu_seqlens, weight, bias=None, residual: bool = False):
-    """Functional form of :class:`VarlenDWConv1dFunction`."""
+    """Functional form of :class:`VarlenDWConv1dFunction`. While ``torch.compile`` is tracing, the call goes
+    through the registered custom ops instead (same kernels), so that callers of this function (the padded-batch
+    door among them) never break the graph."""
+    if torch.compiler.is_compiling():
+        return varlen_dwconv_fwd_op(x, cu_seqlens, weight, bias, residual)
     return VarlenDWConv1dFunction.apply(x, cu_seqlens, weight, bias, residual)
 
 
@@ -272,10 +276,7 @@ class VarlenDWConv1d(nn.Module):
         return padded_dwconv(x, attention_mask, self.weight, self.bias, self.residual, assume_right_padded)
 
     def forward(self, x: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
-        if torch.compiler.is_compiling():
-            # under torch.compile the opaque custom ops keep the graph whole
-            return varlen_dwconv_fwd_op(x, cu_seqlens, self.weight, self.bias, self.residual)
-        return VarlenDWConv1dFunction.apply(x, cu_seqlens, self.weight, self.bias, self.residual)
+        return varlen_dwconv(x, cu_seqlens, self.weight, self.bias, self.residual)
 
     def forward_gated(self, z: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
         """SwiGLU door: ``z = Wi(x)`` of width ``2 * channels`` (x_proj columns, then gate columns);

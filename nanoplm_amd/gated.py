@@ -11,23 +11,23 @@ For a conv placed inside the reference's SwiGLU MLP
 ``gated_varlen_dwconv(z, cu_seqlens, weight, bias)`` takes ``z = self.Wi(x)`` (``[T, 2C]``: x_proj in
 columns ``[0, C)``, gate in ``[C, 2C)``) and returns ``conv(h)`` ``[T, C]`` without ever writing ``h``:
 the forward reads z once and writes y, the backward reads z and dy and writes dz = [d x_proj | d gate],
-dw and db. Shapes the fused kernels are not built for (see ``gated_supported``) run the same HIP
-conv after the gate product is formed with ordinary elementwise ops.
+dw and db. Shapes the fused kernels are not built for (the library says so with its return code) run the
+same HIP conv after the gate product is formed with ordinary elementwise GPU ops.
 """
 from __future__ import annotations
 
 from typing import Optional
 
 import torch
-import torch.nn.functional as F
 
 from . import _lib
-from .dwconv import _DTYPES, _launch_on, _ptr, varlen_dwconv
+from .dwconv import _DTYPES, _launch_on, _ptr, varlen_dwconv_bwd, varlen_dwconv_fwd
 
 
 def gated_supported(z: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the fused kernels take this call (kernel size 3/5/7/9, rows of C*elemsize >= 1 KiB in
-    multiples of 16 bytes, 16-byte aligned contiguous z on a ROCm device)."""
+    """Whether the fused kernels take this call (a kernel size they are built for, rows of C*elemsize >= 1 KiB
+    in multiples of 16 bytes, 16-byte aligned contiguous z on a ROCm device). Informational: the entry
+    points below find out from the library's return code."""
     if not (isinstance(z, torch.Tensor) and z.is_cuda and z.dim() == 2 and z.shape[1] % 2 == 0):
         return False
     if z.dtype not in _DTYPES or weight.dtype not in _DTYPES or not z.is_contiguous() or z.data_ptr() % 16:
@@ -40,6 +40,8 @@ def gated_supported(z: torch.Tensor, weight: torch.Tensor) -> bool:
 def _check(z, cu_seqlens, weight, bias):
     if z.dim() != 2 or z.shape[1] % 2:
         raise ValueError("z must be [T, 2C]: x_proj columns followed by gate columns")
+    if not z.is_cuda:
+        raise RuntimeError(f"gated_varlen_dwconv runs only on a ROCm device (z is on {z.device}); there is no CPU implementation")
     T, C = z.shape[0], z.shape[1] // 2
     if tuple(weight.shape[:1]) != (C,) or weight.dim() != 2:
         raise ValueError(f"weight must be [C={C}, K], got {tuple(weight.shape)}")
@@ -50,8 +52,20 @@ def _check(z, cu_seqlens, weight, bias):
     return T, C, weight.shape[1], cu_seqlens.numel() - 1
 
 
+def _gate_terms(z):
+    """fp32 pieces of h = x_proj * silu(gate): (x_proj, gate * sigmoid(gate), sigmoid(gate), gate)."""
+    u, g = z.chunk(2, dim=-1)
+    uf, gf = u.float(), g.float()
+    sg = torch.sigmoid(gf)
+    return uf, gf * sg, sg, gf
+
+
 def gated_dwconv_fwd(z, cu_seqlens, weight, bias=None, *, residual: bool = False):
-    """Raw fused forward (no autograd): y [T, C] = conv(z[:, :C] * silu(z[:, C:]))."""
+    """Raw forward (no autograd): y [T, C] = conv(z[:, :C] * silu(z[:, C:])).
+
+    Fused kernels where the library has them; a shape it reports as unsupported (other kernel sizes, rows
+    under 1 KiB or not a multiple of 16 bytes, a view that is not 16-byte aligned) forms the gate product
+    with elementwise GPU ops and runs the plain HIP conv on it (h is then rounded once to z's dtype)."""
     T, C, K, S = _check(z, cu_seqlens, weight, bias)
     lib = _lib.load()
     z = z.contiguous()
@@ -63,12 +77,15 @@ def gated_dwconv_fwd(z, cu_seqlens, weight, bias=None, *, residual: bool = False
         rc = lib.nplm_dwconv_gated_fwd(_ptr(z), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(bias), _ptr(y), T, C, K, S,
                                        _DTYPES[z.dtype], _DTYPES[weight.dtype], _lib.RESIDUAL if residual else 0,
                                        dev.stream)
+    if rc == -_lib.EUNSUPPORTED:
+        uf, gs, _, _ = _gate_terms(z)
+        return varlen_dwconv_fwd((uf * gs).to(z.dtype), cu_seqlens, weight, bias, residual=residual)
     _lib.check(rc, "nplm_dwconv_gated_fwd")
     return y
 
 
 def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
-    """Raw fused backward: (dz [T, 2C] in z's dtype, dw [C, K] fp32, db [C] fp32)."""
+    """Raw backward: (dz [T, 2C] in z's dtype, dw [C, K] fp32, db [C] fp32); unsupported shapes as in the forward."""
     T, C, K, S = _check(z, cu_seqlens, weight, None)
     if tuple(dy.shape) != (T, C) or dy.dtype != z.dtype or dy.device != z.device:
         raise ValueError("dy must be [T, C] in z's dtype on z's device")
@@ -77,15 +94,23 @@ def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
     dy = dy.contiguous()
     weight = weight.contiguous()
     act = _DTYPES[z.dtype]
-    dz = torch.empty_like(z)
-    dw = torch.empty((C, K), dtype=torch.float32, device=z.device)
-    db = torch.empty((C,), dtype=torch.float32, device=z.device)
     with _launch_on(z) as dev:
         nbytes = int(lib.nplm_dwconv_gated_bwd_workspace_bytes(T, C, K, act))
-        ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=z.device)
-        rc = lib.nplm_dwconv_gated_bwd(_ptr(z), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(dz), _ptr(dw),
-                                       _ptr(db), _ptr(ws), ws.numel(), T, C, K, S, act, _DTYPES[weight.dtype],
-                                       _lib.RESIDUAL if residual else 0, dev.stream)
+        rc = -_lib.EUNSUPPORTED
+        if nbytes > 0 or T == 0:
+            dz = torch.empty_like(z)
+            dw = torch.empty((C, K), dtype=torch.float32, device=z.device)
+            db = torch.empty((C,), dtype=torch.float32, device=z.device)
+            ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=z.device)
+            rc = lib.nplm_dwconv_gated_bwd(_ptr(z), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(dz), _ptr(dw),
+                                           _ptr(db), _ptr(ws), ws.numel(), T, C, K, S, act, _DTYPES[weight.dtype],
+                                           _lib.RESIDUAL if residual else 0, dev.stream)
+    if rc == -_lib.EUNSUPPORTED:
+        uf, gs, sg, gf = _gate_terms(z)
+        dh, dw, db = varlen_dwconv_bwd((uf * gs).to(z.dtype), dy, cu_seqlens, weight, residual=residual)
+        dhf = dh.float()
+        dz = torch.cat((dhf * gs, dhf * uf * sg * (1.0 + gf * (1.0 - sg))), dim=-1).to(z.dtype)
+        return dz, dw, db
     _lib.check(rc, "nplm_dwconv_gated_bwd")
     return dz, dw, db
 
@@ -116,18 +141,11 @@ def gated_varlen_dwconv(z: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch
                         bias: Optional[torch.Tensor] = None, residual: bool = False) -> torch.Tensor:
     """``conv(z[:, :C] * silu(z[:, C:]))`` over packed sequences, ``[T, 2C] -> [T, C]``.
 
-    Fused kernels where they are built (``gated_supported``); otherwise the gate product is formed by
-    elementwise ops and the plain HIP conv runs on it (same result to rounding)."""
+    Under ``torch.compile`` the call goes through the registered custom ops (opaque to the tracer, no graph
+    break, any shape); otherwise through the autograd Function. Both run the same two raw entry points."""
     if torch.compiler.is_compiling():
-        # static shapes under torch.compile: a contiguous [T, 2C] activation of a supported width takes the
-        # registered fused ops (opaque to the tracer, no graph break)
-        if z.dim() == 2 and z.is_contiguous() and weight.shape[1] in (3, 5, 7, 9) and \
-                (z.shape[1] // 2 * z.element_size()) % 16 == 0 and z.shape[1] // 2 * z.element_size() >= 1024:
-            return gated_dwconv_fwd_op(z, cu_seqlens, weight, bias, residual)
-    elif gated_supported(z, weight):
-        return GatedVarlenDWConv1dFunction.apply(z, cu_seqlens, weight, bias, residual)
-    x_proj, gate = z.chunk(2, dim=-1)
-    return varlen_dwconv((F.silu(gate) * x_proj).contiguous(), cu_seqlens, weight, bias, residual)
+        return gated_dwconv_fwd_op(z, cu_seqlens, weight, bias, residual)
+    return GatedVarlenDWConv1dFunction.apply(z, cu_seqlens, weight, bias, residual)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -53,6 +53,35 @@ def assert_red_close(got, ref64, what, atol=DWDB_ATOL):
     return err
 
 
+def error_stats(got, ref64, dtype=None):
+    """What the parity tables report for one tensor: max-abs and max-rel error (rel over |ref| > 1e-3), and for
+    bf16 how many elements have |ref| >= 8 (where one bf16 rounding exceeds 2e-2) with their max-abs error."""
+    got = got.detach().cpu().double()
+    err = (got - ref64).abs()
+    big = ref64.abs() > 1e-3
+    out = {"max_abs": float(err.max()), "max_rel": float((err[big] / ref64[big].abs()).max()) if big.any() else 0.0,
+           "max_ref": float(ref64.abs().max())}
+    if dtype == torch.bfloat16:
+        large = ref64.abs() >= 8.0
+        out["n_ref_ge_8"] = int(large.sum())
+        out["max_abs_ref_ge_8"] = float(err[large].max()) if large.any() else 0.0
+        out["max_abs_ref_lt_8"] = float(err[~large].max()) if (~large).any() else 0.0
+    return out
+
+
+def record_parity(name, stats):
+    """Keep the parity magnitudes of a run as gpurun_out/parity_<name>.json (best effort: the figures are also printed)."""
+    import json
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    try:
+        os.makedirs(os.path.join(root, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(root, "gpurun_out", f"parity_{name}.json"), "w") as f:
+            json.dump(stats, f, indent=1)
+    except OSError:
+        pass
+
+
 @functools.lru_cache(maxsize=2)
 def workload_with_oracle(index, T=None, C=None):
     """(workload on CPU, y64, dx64, dw64, db64) with the C oracle; dy is always generated."""

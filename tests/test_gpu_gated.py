@@ -84,20 +84,102 @@ def test_gated_autograd_matches_the_unfused_composition_and_is_deterministic():
     assert torch.equal(y3, y1) and torch.equal(z3.grad, z1.grad) and torch.equal(w3.grad, w1.grad)
 
 
+def _composed_case_matches(z, cu, w, b, dy, what):
+    """A shape without fused kernels: the raw entry points and the autograd surface compose the unfused ops; h is
+    rounded to z's dtype on this route, so bf16 gets a bf16-sized allowance on top of the conv's own tolerance."""
+    y64, dz64, dw64, db64 = O.ref_gated_dwconv_grads(z, cu, w, b, dy, torch.float64)
+    zd, cud, wd, bd, dyd = (t.to(DEV) for t in (z, cu, w, b, dy))
+    z1 = zd.clone().requires_grad_(True)
+    w1 = wd.clone().requires_grad_(True)
+    b1 = bd.clone().requires_grad_(True)
+    y = npa.gated_varlen_dwconv(z1, cud, w1, b1)
+    y.backward(dyd)
+    tol = 4e-2 if z.dtype == torch.bfloat16 else 1e-4
+    scale = lambda r: max(1.0, float(r.abs().max()))
+    assert float((y.detach().cpu().double() - y64).abs().max()) <= tol * scale(y64), what
+    assert float((z1.grad.cpu().double() - dz64).abs().max()) <= tol * scale(dz64), what
+    assert float((w1.grad.cpu().double() - dw64).abs().max()) <= 2 * tol * scale(dw64), what
+    assert float((b1.grad.cpu().double() - db64).abs().max()) <= 2 * tol * scale(db64), what
+    return zd, cud, wd, bd, dyd
+
+
 def test_unsupported_shapes_compose_and_the_abi_says_so():
     z, cu, w, b, dy = _case([5, 40, 3], 100, 7, torch.bfloat16, torch.bfloat16, seed=1)     # 200-byte rows
-    zd, cud, wd, bd = z.to(DEV), cu.to(DEV), w.to(DEV), b.to(DEV)
+    zd, cud, wd, bd, _ = _composed_case_matches(z, cu, w, b, dy, "200-byte rows")
     assert not npa.gated_supported(zd, wd)
-    y = npa.gated_varlen_dwconv(zd, cud, wd, bd)
-    y64 = O.ref_gated_dwconv_grads(z, cu, w, b, None)
-    assert float((y.cpu().double() - y64).abs().max()) <= 3e-2      # h is rounded to bf16 on this route
     lib = _lib.load()
     out = torch.empty(48, 100, device=DEV, dtype=torch.bfloat16)
     rc = lib.nplm_dwconv_gated_fwd(zd.data_ptr(), cud.data_ptr(), wd.data_ptr(), None, out.data_ptr(), 48, 100, 7, 3, 1, 1, 0,
                                    torch.cuda.current_stream().cuda_stream)
     assert rc == -_lib.EUNSUPPORTED and "gated" in _lib.strerror(rc)
-    z11, _, w11, b11, _ = _case([30, 30], 1024, 11, torch.bfloat16, torch.bfloat16, seed=2)  # K = 11
-    assert not npa.gated_supported(z11.to(DEV), w11.to(DEV))
+    c11 = _case([30, 30], 1024, 11, torch.bfloat16, torch.bfloat16, seed=2)  # K = 11
+    assert not npa.gated_supported(c11[0].to(DEV), c11[2].to(DEV))
+    _composed_case_matches(*c11, "K=11")
+    _composed_case_matches(*_case([30, 7, 30], 512, 13, torch.float32, torch.float32, seed=3), "K=13 fp32")
+
+
+def test_offset_view_of_z_composes_instead_of_failing():
+    """z that is contiguous but starts 8 bytes off a 16-byte boundary: the fused kernels decline, the call still works,
+    eagerly and through the registered ops."""
+    z, cu, w, b, dy = _case([40, 3, 200, 13], 1024, 7, torch.bfloat16, torch.bfloat16, seed=5)
+    T = z.shape[0]
+    buf = torch.zeros(T * 2048 + 8, dtype=torch.bfloat16, device=DEV)
+    zv = buf[4:4 + T * 2048].view(T, 2048)
+    zv.copy_(z)
+    assert zv.is_contiguous() and zv.data_ptr() % 16 == 8
+    cud, wd, bd, dyd = (t.to(DEV) for t in (cu, w, b, dy))
+    y_al = npa.gated_dwconv_fwd(z.to(DEV), cud, wd, bd)
+    y = npa.gated_dwconv_fwd(zv, cud, wd, bd)
+    y_op = npa.gated_dwconv_fwd_op(zv, cud, wd, bd)
+    assert torch.equal(y, y_op)
+    def close(a, b):      # h is rounded to bf16 on the composed route: about one bf16 rounding of the result
+        a, b = a.float(), b.float()
+        return bool(((a - b).abs() <= 2.0 ** -6 * b.abs() + 3e-2).all())
+
+    assert close(y, y_al)
+    dz, dw, db = npa.gated_dwconv_bwd(zv, dyd, cud, wd)
+    dz_al, dw_al, db_al = npa.gated_dwconv_bwd(z.to(DEV), dyd, cud, wd)
+    assert close(dz, dz_al)
+    torch.testing.assert_close(dw, dw_al, rtol=2e-2, atol=0.5)
+    torch.testing.assert_close(db, db_al, rtol=1e-5, atol=1e-3)
+
+
+@pytest.mark.parametrize("C,K", [(2048, 31), (1024, 11), (100, 7)])
+def test_every_gated_shape_compiles_without_graph_breaks(C, K):
+    """Intermediate width with the long kernel, a kernel size without fused kernels and narrow rows: under
+    torch.compile(fullgraph=True) each is one opaque op, whichever route the library takes inside it."""
+    print(f"[case] gated compile C={C} K={K}", flush=True)
+    z, cu, w, b, dy = _case([40, 3, 200, 13, 300], C, K, torch.bfloat16, torch.bfloat16, seed=C + K)
+    zd, cud, dyd = z.to(DEV), cu.to(DEV), dy.to(DEV)
+    conv = npa.VarlenDWConv1d(C, K, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        conv.weight.copy_(w.to(DEV))
+        conv.bias.copy_(b.to(DEV))
+
+    class MLPTail(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = conv
+
+        def forward(self, zz, cc):
+            return self.conv.forward_gated(zz, cc)
+
+    def run(mod):
+        conv.zero_grad()
+        zin = zd.clone().requires_grad_(True)
+        y = mod(zin, cud)
+        y.backward(dyd)
+        return y.detach(), zin.grad, conv.weight.grad.clone(), conv.bias.grad.clone()
+
+    m = MLPTail()
+    eager = run(m)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(m, backend="aot_eager", fullgraph=True, dynamic=False))
+    for a, bb in zip(eager, compiled):
+        assert torch.equal(a, bb)
+    y64, dz64, _, _ = O.ref_gated_dwconv_grads(z, cu, w, b, dy, torch.float64)
+    assert float((eager[0].cpu().double() - y64).abs().max()) <= 4e-2 * max(1.0, float(y64.abs().max()))
+    assert float((eager[1].cpu().double() - dz64).abs().max()) <= 4e-2 * max(1.0, float(dz64.abs().max()))
 
 
 def test_gated_ops_pass_opcheck_and_compile_without_graph_breaks():

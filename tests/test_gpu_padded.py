@@ -105,3 +105,37 @@ def test_flat_weight_module_trains_like_the_2d_one():
     # zero-initialised residual block is the identity
     z = npa.VarlenDWConv1d(128, 7, residual=True, init="zero", device=DEV)
     assert torch.equal(z(x, cu), x)
+
+
+def test_padded_door_compiles_without_graph_breaks():
+    """forward_padded inside a compiled model (torch.compile(dynamic=False), pure_pipeline.py:519-524): the call
+    reaches the registered custom ops, so fullgraph=True holds, forward and backward."""
+    lens = [37, 128, 0, 1, 90, 128, 5]
+    x, mask, w, bias = _padded_case(lens, 128, 1024, 7, torch.bfloat16, seed=3)
+    conv = npa.VarlenDWConv1d(1024, 7, residual=True, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        conv.weight.copy_(w.to(DEV))
+        conv.bias.copy_(bias.to(DEV))
+    xd, md = x.to(DEV), mask.to(DEV)
+
+    class Door(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = conv
+
+        def forward(self, xx, mm):
+            return self.conv.forward_padded(xx, mm)
+
+    def run(mod):
+        conv.zero_grad()
+        xin = xd.clone().requires_grad_(True)
+        y = mod(xin, md)
+        y.float().square().sum().backward()
+        return y.detach(), xin.grad, conv.weight.grad.clone(), conv.bias.grad.clone()
+
+    door = Door()
+    eager = run(door)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(door, backend="aot_eager", fullgraph=True, dynamic=False))
+    for a, b in zip(eager, compiled):
+        assert torch.equal(a, b)

@@ -13,7 +13,7 @@ from nanoplm_amd import _lib
 from nanoplm_amd.workloads import cu_from_lengths, make_workload, static_packed_cu
 from oracle import dwconv_ref as O
 
-from gpu_util import assert_act_close, assert_red_close, workload_with_oracle
+from gpu_util import assert_act_close, assert_red_close, error_stats, record_parity, workload_with_oracle
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -45,6 +45,9 @@ def test_configuration_matches_oracle(index):
     e_db = assert_red_close(db, db64, f"cfg{index} db")
     print(f"[parity] cfg{index} T={wl.T} C={wl.C} K={wl.K} S={wl.S} {wl.dtype}: max-abs y {e_y:.3e} dx {e_dx:.3e} "
           f"dw {e_dw:.3e} (max|dw| {float(dw64.abs().max()):.1f}) db {e_db:.3e}", flush=True)
+    record_parity(f"cfg{index}", {"workload": wl.name, "T": wl.T, "C": wl.C, "K": wl.K, "S": wl.S,
+                                  "y": error_stats(y, y64, wl.dtype), "dx": error_stats(dx, dx64, wl.dtype),
+                                  "dw": error_stats(dw, dw64), "db": error_stats(db, db64)})
     # run-to-run determinism: bit-identical outputs, reductions included
     y2, dx2, dw2, db2 = _run_all(d)
     assert torch.equal(y, y2) and torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.equal(db, db2)

@@ -62,13 +62,17 @@ def test_random_case_matches_oracle(case):
     tune = _lib.Tuning(algo=algo) if algo else None
     xd, dyd, wd, cud = x.to(DEV), dy.to(DEV), w.to(DEV), cu.to(DEV)
     bd = None if b is None else b.to(DEV)
+    def run(t):
+        return (npa.varlen_dwconv_fwd(xd, cud, wd, bd, residual=residual, tuning=t),
+                *npa.varlen_dwconv_bwd(xd, dyd, cud, wd, residual=residual, tuning=t))
+
     try:
-        y = npa.varlen_dwconv_fwd(xd, cud, wd, bd, residual=residual, tuning=tune)
-        dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, residual=residual, tuning=tune)
+        y, dx, dw, db = run(tune)
     except RuntimeError as e:
-        if algo == 2 and "not available" in str(e):
-            pytest.skip("LDS-staged kernels are not built for this shape")   # narrow rows, other K
-        raise
+        if not (algo == 2 and "not available" in str(e)):
+            raise
+        # no LDS-staged kernel for this shape (narrow rows, other kernel sizes): the case runs on the library's own choice
+        y, dx, dw, db = run(None)
     y64 = O.c_oracle_fwd(x, cu, w, b, residual=residual)
     dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w, residual=residual)
     assert_act_close(y, y64, dt, "y")
