@@ -56,7 +56,7 @@ extern "C" {
 
 /* argument errors (returned negated: -NPLM_DWCONV_E...) */
 #define NPLM_DWCONV_ENULL      1  /* a required pointer is NULL */
-#define NPLM_DWCONV_ESHAPE     2  /* T < 0, T > 2^31 - 2^20 - 1, C < 1, S < 0, or C*K too large */
+#define NPLM_DWCONV_ESHAPE     2  /* T < 0, T > 2^31 - 2^20 - 1, C < 1, S < 0, or C*K >= 2^28 */
 #define NPLM_DWCONV_EKSIZE     3  /* K < 1, K even, or K > NPLM_DWCONV_MAX_K */
 #define NPLM_DWCONV_EDTYPE     4  /* unknown act_dtype / w_dtype */
 #define NPLM_DWCONV_EALIGN     5  /* activation pointer not aligned to its element size */
@@ -64,6 +64,7 @@ extern "C" {
 #define NPLM_DWCONV_ECU        7  /* check_cu: cu[0] != 0, cu decreasing, or cu[S] != T */
 #define NPLM_DWCONV_EFLAGS     9  /* unknown bits set in `flags` (8 is used by the internal tuning interface) */
 #define NPLM_DWCONV_EUNSUPPORTED 10 /* gated entry points: shape outside what the fused kernels are built for */
+#define NPLM_DWCONV_ESCRATCH   11 /* nplm_dwconv_bwd_static: the partial sums do not fit the static scratch */
 
 /* flags of the _ex entry points */
 #define NPLM_DWCONV_RESIDUAL 1u   /* fuse the residual connection: y = x + conv(x), dx = dy + conv^T(dy) */
@@ -127,6 +128,26 @@ int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const v
                        void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,
                        int64_t T, int32_t C, int32_t K, int32_t S,
                        int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
+
+/*
+ * Backward for callers that cannot allocate: code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc, which therefore cannot produce the workspace nplm_dwconv_bwd_ex
+ * asks for. No counterpart in the reference. Same arguments, kernels and results (bit for bit) as
+ * nplm_dwconv_bwd_ex, minus the workspace: the dw/db partial sums go to a scratch array of
+ * NPLM_DWCONV_STATIC_SCRATCH_BYTES that lives in the library's own device image, one copy per GPU,
+ * held until the process ends. The call allocates and frees nothing. Its first use on a device looks
+ * the array's address up (hipGetSymbolAddress) and keeps it, so make one call per device outside any
+ * capture. Shapes whose partial sums need more than the array holds (C*(K+1) above 4 Mi elements)
+ * return -NPLM_DWCONV_ESCRATCH and launch nothing. Every call on a GPU shares that GPU's array: two
+ * calls that overlap in time on one GPU (different streams, or threads) race on it and corrupt each
+ * other's dw/db; calls on one stream, or otherwise ordered, are safe. Nothing in the array has to be
+ * cleared between calls (every slab a call reads it has fully written first).
+ */
+#define NPLM_DWCONV_STATIC_SCRATCH_BYTES (16u << 20)
+int nplm_dwconv_bwd_static(const void* x, const void* dy, const int32_t* cu, const void* w,
+                           void* dx, float* dw, float* db,
+                           int64_t T, int32_t C, int32_t K, int32_t S,
+                           int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
  * Gated variants: the conv over h = x_proj * silu(gate) with the gate product fused into the conv's

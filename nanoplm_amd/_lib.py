@@ -15,6 +15,8 @@ F32 = 0
 BF16 = 1
 RESIDUAL = 1    # NPLM_DWCONV_RESIDUAL
 EUNSUPPORTED = 10   # NPLM_DWCONV_EUNSUPPORTED
+ESCRATCH = 11       # NPLM_DWCONV_ESCRATCH
+STATIC_SCRATCH_BYTES = 16 << 20   # NPLM_DWCONV_STATIC_SCRATCH_BYTES
 
 # every symbol include/nplm_dwconv.h declares
 PUBLIC_SYMBOLS = (
@@ -25,6 +27,7 @@ PUBLIC_SYMBOLS = (
     "nplm_dwconv_bwd_workspace_bytes",
     "nplm_dwconv_bwd",
     "nplm_dwconv_bwd_ex",
+    "nplm_dwconv_bwd_static",
     "nplm_dwconv_gated_fwd",
     "nplm_dwconv_gated_bwd_workspace_bytes",
     "nplm_dwconv_gated_bwd",
@@ -71,6 +74,8 @@ def load():
     lib.nplm_dwconv_bwd.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_ex.argtypes = bwd_args[:-1] + [ctypes.c_uint32, vp]
     lib.nplm_dwconv_bwd_ex.restype = ctypes.c_int
+    lib.nplm_dwconv_bwd_static.argtypes = bwd_args[:7] + bwd_args[9:-1] + [ctypes.c_uint32, vp]
+    lib.nplm_dwconv_bwd_static.restype = ctypes.c_int
     lib.nplm_dwconv_gated_fwd.argtypes = fwd_args[:-1] + [ctypes.c_uint32, vp]
     lib.nplm_dwconv_gated_fwd.restype = ctypes.c_int
     lib.nplm_dwconv_gated_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]

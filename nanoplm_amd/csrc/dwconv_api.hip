@@ -10,15 +10,22 @@
 #include <limits.h>
 #include <stdlib.h>
 
+#include <atomic>
 #include <vector>
 
 #include "../../include/nplm_dwconv.h"
 #include "dwconv_internal.h"
 
+// Scratch of nplm_dwconv_bwd_static: the dw/db partial-sum slabs of one backward call, for callers that
+// cannot hand in a workspace they allocated. One copy per GPU, held until the process ends. Host code
+// never uses this name as an address: static_scratch_for_current_device() asks the runtime where the
+// current device's copy lives and the kernels are given that pointer.
+static __device__ __align__(256) unsigned char scratch[NPLM_DWCONV_STATIC_SCRATCH_BYTES];
+
 namespace nplm {
 namespace {
 
-constexpr int kVersion = 100;   // 0.1.0
+constexpr int kVersion = 101;   // 0.1.1
 
 // MI355X: 256 CUs in 8 XCDs. Geometry is a pure function of the problem size so that the
 // reduction order (and with it every output bit) is reproducible.
@@ -479,6 +486,26 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     return 0;
 }
 
+// Device address of `scratch` on the current device, looked up once per device and kept.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+hipError_t static_scratch_for_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);   // every thread finds the same address
+    }
+    *out = p;
+    return hipSuccess;
+}
+
 }  // namespace
 }  // namespace nplm
 
@@ -575,7 +602,7 @@ const char* nplm_dwconv_strerror(int code) {
     if (code > 0) return hipGetErrorString((hipError_t)code);
     switch (-code) {
         case NPLM_DWCONV_ENULL: return "nplm_dwconv: a required pointer is NULL";
-        case NPLM_DWCONV_ESHAPE: return "nplm_dwconv: invalid sizes (need 0 <= T <= INT32_MAX, C >= 1, S >= 0)";
+        case NPLM_DWCONV_ESHAPE: return "nplm_dwconv: invalid sizes (need 0 <= T <= 2^31 - 2^20 - 1, C >= 1, S >= 0, C*K < 2^28)";
         case NPLM_DWCONV_EKSIZE: return "nplm_dwconv: kernel size must be odd and in [1, 255]";
         case NPLM_DWCONV_EDTYPE: return "nplm_dwconv: unknown element type (0 = fp32, 1 = bf16)";
         case NPLM_DWCONV_EALIGN: return "nplm_dwconv: pointer not aligned to its element size";
@@ -583,6 +610,7 @@ const char* nplm_dwconv_strerror(int code) {
         case NPLM_DWCONV_ECU: return "nplm_dwconv: cu_seqlens must start at 0, be non-decreasing and end at T";
         case NPLM_DWCONV_EFLAGS: return "nplm_dwconv: unknown bits set in flags";
         case NPLM_DWCONV_EUNSUPPORTED: return "nplm_dwconv: shape not supported by the fused gated kernels";
+        case NPLM_DWCONV_ESCRATCH: return "nplm_dwconv: the dw/db partial sums of this shape do not fit the library's static scratch (16 MiB); use nplm_dwconv_bwd_ex with a caller-owned workspace";
         case NPLM_DWCONV_ETUNING: return "nplm_dwconv: geometry override not available in this build";
     }
     return "nplm_dwconv: unknown error code";
@@ -647,6 +675,23 @@ int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const v
                        int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
     return bwd_impl(x, dy, cu, w, dx, dw, db, workspace, workspace_bytes, T, C, K, S, act_dtype, w_dtype, flags,
                     stream, nullptr);
+}
+
+int nplm_dwconv_bwd_static(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw,
+                           float* db, int64_t T, int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype,
+                           uint32_t flags, void* stream) {
+    const int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    void* ws = nullptr;
+    size_t ws_bytes = 0;
+    if (T > 0 && (dw || db)) {
+        // the same number of slabs nplm_dwconv_bwd_ex would ask its caller for
+        ws_bytes = nplm_dwconv_bwd_workspace_bytes(T, C, K, act_dtype);
+        if (ws_bytes == 0 || ws_bytes > (size_t)NPLM_DWCONV_STATIC_SCRATCH_BYTES) return -NPLM_DWCONV_ESCRATCH;
+        const hipError_t e = static_scratch_for_current_device(&ws);
+        if (e != hipSuccess) return (int)e;
+    }
+    return bwd_impl(x, dy, cu, w, dx, dw, db, ws, ws_bytes, T, C, K, S, act_dtype, w_dtype, flags, stream, nullptr);
 }
 
 int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, const void* w, void* dx, float* dw,
