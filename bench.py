@@ -6,8 +6,12 @@
 A step is one forward plus one backward (dx, dweight, dbias) of the configured workload through the
 C ABI of libnplm_dwconv.so, with every input already resident in HBM. The default workload is
 configuration 3 of nanoplm_amd.workloads (T=131072 packed tokens, C=1024, K=7, bf16), the one the
-headline metric is quoted on. Three input/output sets (> 256 MB each) are rotated so no step reads
-a tensor that is still in the Infinity Cache.
+headline metric is quoted on. Four input/output sets (> 256 MB each) are rotated, and the backward of a
+step works on the set two places away from the forward's, so that no kernel reads a tensor that an
+earlier kernel left in the 256 MB Infinity Cache: at least two other kernels (>= 1.3 GB of traffic) run
+between two touches of the same tensor, as in a training step, where a layer's backward runs long
+after its forward. (ms_per_step_same_tensors is the same loop with forward and backward on one set, where
+the backward finds part of x still cached; informational.)
 
 Order of one run: an untimed pre-warm (the same forward + backward launches for --prewarm-ms, so that
 the GPU has reached its steady clocks and every buffer has been touched before anything is timed),
@@ -162,7 +166,8 @@ def main():
     d = wl.to(dev)
     T, C, K, S = wl.T, wl.C, wl.K, wl.S
     fwd_bwd = wl.passes == "fwd+bwd"
-    NSET = 3
+    NSET = 4
+    BWD_SHIFT = 2          # the backward of step i uses set (i + BWD_SHIFT) % NSET
     if args.gated and not fwd_bwd:
         sys.exit("--gated needs a forward+backward configuration (3, 4 or 5)")
     xs = [d.x] + [torch.randn(T, C, device=dev).to(wl.dtype) for _ in range(NSET - 1)]
@@ -190,8 +195,8 @@ def main():
         _lib.check(lib.nplm_dwconv_fwd_ex(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(),
                                           ys[j].data_ptr(), T, C, K, S, act, act, flags, stream), "nplm_dwconv_fwd_ex")
 
-    def bwd(i, t=None):
-        j = i % NSET
+    def bwd(i, t=None, shift=BWD_SHIFT):
+        j = (i + shift) % NSET
         args_ = (xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(),
                  db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act)
         if args.gated:
@@ -231,6 +236,16 @@ def main():
         rep_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
     ms_per_step = statistics.median(rep_ms)
     tokens_per_s = T / (ms_per_step / 1e3)
+    same_ms = []
+    if fwd_bwd:      # informational: forward and backward of a step on the same tensors
+        for _ in range(5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                fwd(i)
+                bwd(i, shift=0)
+            torch.cuda.synchronize()
+            same_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
 
     # ---- per-kernel durations with HIP events on the launch stream ---------------------------------
     # The same step sequence as the timed loop above, launched back to back without host
@@ -299,11 +314,12 @@ def main():
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_min": min(rep_ms), "reps": len(rep_ms),
         "ms_per_step_reps": [round(v, 5) for v in rep_ms], "prewarm_ms": prewarm_ms, "prewarm_steps": prewarm_steps,
+        "ms_per_step_same_tensors": statistics.median(same_ms) if same_ms else None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
         "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
-                   "rotating_sets": NSET, "residual": bool(args.residual), "gated": bool(args.gated)},
+                   "rotating_sets": NSET, "backward_set_shift": BWD_SHIFT if fwd_bwd else None, "residual": bool(args.residual), "gated": bool(args.gated)},
         "step_algorithmic_bytes": step_bytes,
         "step_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,

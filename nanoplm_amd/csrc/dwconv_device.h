@@ -54,6 +54,39 @@ __device__ __forceinline__ rsrc_t rows_rsrc(const void* tensor, int row0, int T,
     return make_rsrc(reinterpret_cast<const char*>(tensor) + (size_t)row0 * row_bytes, n);
 }
 
+// Cache policy of the activation streams: the aux operand of the MUBUF builtins on gfx950 (bit 0 = sc0,
+// bit 1 = nt, bit 4 = sc1). x, dy, y and dx are each touched once per call, plus the K-1 halo rows a
+// neighbouring tile re-reads within the same round of tiles. Measured on MI355X at T=131072, C=1024, K=7, bf16
+// (wall-clock forward+backward step on tensors no earlier kernel left in a cache; 244.8 us with no hints):
+//   stores of y and dx non-temporal                      235.3 us (forward 95.0 -> 90.0, backward+finalize 149.5 -> 146.2)
+//   + backward loads of rows only one tile reads, nt     234.8 us (backward+finalize 144.0); the Infinity Cache is then
+//                                                         left to other tensors (with x still cached from the forward
+//                                                         of the same step: 223.7 us)
+//   backward x loads nt but dy loads plain               240.0 us
+//   forward loads nt (all rows, or all but halo rows)    257.0 / 239.9 us: the forward slows from 90 to 100-103 us
+//   sc0/sc1 variants of either                           no better than nt alone (235.2 - 237.7 us)
+// The defaults below are the second line. (A plain copy kernel gains more from nt loads: 5.73 -> 6.27 TB/s.)
+#ifndef NPLM_LOAD_AUX
+#define NPLM_LOAD_AUX 0            // rows a neighbouring tile stages as well, and every load of the forward
+#endif
+#ifndef NPLM_LOAD_AUX_ONCE_FWD
+#define NPLM_LOAD_AUX_ONCE_FWD NPLM_LOAD_AUX
+#endif
+#ifndef NPLM_LOAD_AUX_ONCE_BWD
+#define NPLM_LOAD_AUX_ONCE_BWD 2   // nt
+#endif
+#ifndef NPLM_LOAD_AUX_ONCE_BWDX
+#define NPLM_LOAD_AUX_ONCE_BWDX NPLM_LOAD_AUX_ONCE_BWD
+#endif
+#ifndef NPLM_STORE_AUX
+#define NPLM_STORE_AUX 2           // nt
+#endif
+constexpr int kLoadAux = NPLM_LOAD_AUX;
+constexpr int kLoadAuxOnceFwd = NPLM_LOAD_AUX_ONCE_FWD;   // LDS-staged forward: x rows only one tile reads
+constexpr int kLoadAuxOnceBwd = NPLM_LOAD_AUX_ONCE_BWD;   // LDS-staged backward: dy rows only one tile reads
+constexpr int kLoadAuxOnceBwdX = NPLM_LOAD_AUX_ONCE_BWDX; // LDS-staged backward: x rows (no halo)
+constexpr int kStoreAux = NPLM_STORE_AUX;
+
 // ---------------------------------------------------------------------------------------------
 // RowVec: VEC adjacent channels of one row, as stored in memory.
 // ---------------------------------------------------------------------------------------------
@@ -76,14 +109,14 @@ template <int VEC> struct RowVec<true, VEC> {
         else { *reinterpret_cast<uint32_t*>(p) = d[0]; }
     }
     __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) {
-        if constexpr (NDW == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w; }
-        else if constexpr (NDW == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); d[0] = t.x; d[1] = t.y; }
-        else { d[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0); }
+        if constexpr (NDW == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, kLoadAux); d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w; }
+        else if constexpr (NDW == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, kLoadAux); d[0] = t.x; d[1] = t.y; }
+        else { d[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, kLoadAux); }
     }
     __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const {
-        if constexpr (NDW == 4) { u32x4 t = {d[0], d[1], d[2], d[3]}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, 0); }
-        else if constexpr (NDW == 2) { u32x2 t = {d[0], d[1]}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, 0); }
-        else { __builtin_amdgcn_raw_buffer_store_b32(d[0], r, voff, soff, 0); }
+        if constexpr (NDW == 4) { u32x4 t = {d[0], d[1], d[2], d[3]}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, kStoreAux); }
+        else if constexpr (NDW == 2) { u32x2 t = {d[0], d[1]}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, kStoreAux); }
+        else { __builtin_amdgcn_raw_buffer_store_b32(d[0], r, voff, soff, kStoreAux); }
     }
     __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
 #pragma unroll
@@ -99,8 +132,8 @@ template <> struct RowVec<true, 1> {
     uint16_t h;
     __device__ __forceinline__ void load(const char* p) { h = *reinterpret_cast<const uint16_t*>(p); }
     __device__ __forceinline__ void store(char* p) const { *reinterpret_cast<uint16_t*>(p) = h; }
-    __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) { h = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0); }
-    __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const { __builtin_amdgcn_raw_buffer_store_b16(h, r, voff, soff, 0); }
+    __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) { h = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, kLoadAux); }
+    __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const { __builtin_amdgcn_raw_buffer_store_b16(h, r, voff, soff, kStoreAux); }
     __device__ __forceinline__ void to_f32(float (&f)[1]) const { f[0] = bf16_to_f32(h); }
     __device__ __forceinline__ void from_f32(const float (&f)[1]) { h = f32_to_bf16(f[0]); }
 };
@@ -120,14 +153,14 @@ template <int VEC> struct RowVec<false, VEC> {
         else { *reinterpret_cast<float*>(p) = v[0]; }
     }
     __device__ __forceinline__ void bload(rsrc_t r, int voff, int soff) {
-        if constexpr (VEC == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w); }
-        else if constexpr (VEC == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); }
-        else { v[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0)); }
+        if constexpr (VEC == 4) { u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, kLoadAux); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); v[2] = __uint_as_float(t.z); v[3] = __uint_as_float(t.w); }
+        else if constexpr (VEC == 2) { u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, kLoadAux); v[0] = __uint_as_float(t.x); v[1] = __uint_as_float(t.y); }
+        else { v[0] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, kLoadAux)); }
     }
     __device__ __forceinline__ void bstore(rsrc_t r, int voff, int soff) const {
-        if constexpr (VEC == 4) { u32x4 t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, 0); }
-        else if constexpr (VEC == 2) { u32x2 t = {__float_as_uint(v[0]), __float_as_uint(v[1])}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, 0); }
-        else { __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[0]), r, voff, soff, 0); }
+        if constexpr (VEC == 4) { u32x4 t = {__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])}; __builtin_amdgcn_raw_buffer_store_b128(t, r, voff, soff, kStoreAux); }
+        else if constexpr (VEC == 2) { u32x2 t = {__float_as_uint(v[0]), __float_as_uint(v[1])}; __builtin_amdgcn_raw_buffer_store_b64(t, r, voff, soff, kStoreAux); }
+        else { __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v[0]), r, voff, soff, kStoreAux); }
     }
     __device__ __forceinline__ void to_f32(float (&f)[VEC]) const {
 #pragma unroll

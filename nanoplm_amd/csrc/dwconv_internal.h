@@ -134,20 +134,25 @@ constexpr int default_unroll(bool bwd, int K, int vec) {
 }
 // Kernel sizes the LDS-staged kernels are built for.
 constexpr bool lds_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 15 || K == 31; }
-// Default shapes: a block owns 1 KiB of every row of a 32-row tile.
+// Default shapes: a block owns 1 KiB of every row of a tile of about 32 rows.
 //   forward : 2 wave-columns x 8 bytes per lane, 4 row groups of 8 rows, 4 loader waves; two x tiles of
 //             32 + K-1 rows (76 KiB of LDS at K = 7).
-//   backward: 4 wave-columns x 4 bytes per lane, 2 row groups of 16 rows, 3 loader waves; two
-//             (dy tile of 32 + K-1 rows, x tile of 32 rows) pairs = 140 KiB of the 160 KiB a CU has.
-//             Four bytes per lane keep the 16-row register tile (dx accumulators + x rows + weights + dw/db)
-//             in the registers 11 waves leave (168; K = 9 in bf16 needs more than 128).
+//   backward: 4 wave-columns x 4 bytes per lane, 3 row groups of 10 rows, 4 loader waves (16 waves, the most a
+//             block can have); two (dy tile of 30 + K-1 rows, x tile of 30 rows) pairs = 132 KiB of the 160 KiB a
+//             CU has. The backward issues 20 vector-ALU instructions per element (14 are the FMAs of dx and dw),
+//             about 68 us per SIMD at the headline shape, so the compute waves need company to hide their LDS
+//             latency: with 12 of them (3 per SIMD) backward + finalize takes 138.8 us where 8 waves of 16 rows
+//             with 3 loader waves took 144.3 us (T=131072, C=1024, K=7, bf16; rows per wave 9 .. 12: 138.0 - 138.9 us;
+//             3 loader waves: 146.2 us; 2: 155.0 us; 8 bytes per lane spill: 169 us and worse).
+//             A third tile buffer was measured slower: 3 x 16-row tiles 179 us against 165 us for 2 x 16-row, 3 x
+//             22-row tiles 162 us. So was the forward's boundary mailbox (loader waves running the lookup):
+//             141.9 us against 138.8 us.
 // Measured at T=131072, C=1024, K=7, bf16 against 16-row tiles on 2 KiB column blocks (the same bytes per
-// tile, more halo rows per output row, twice the barriers): forward 98 -> 95 us, backward + finalize
-// 155 -> 151 us; more loader waves than these are slower (backward with 4: 153, with 5: 155 us).
+// tile, more halo rows per output row, twice the barriers), before the cache-policy hints: forward 98 -> 95 us.
 constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
     if (K >= 15)   // long kernels: 32-row tiles of 16-row waves, so that tile + K-1 halo rows still fit twice
         return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 2, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
-    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 3, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 4, 2, 4, 2};
+    return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 10, 3, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 4, 2, 4, 2};
 }
 constexpr int kLdsDefaultCb = 1024;
 // Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block

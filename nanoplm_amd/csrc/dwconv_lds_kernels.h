@@ -121,9 +121,19 @@ struct LdsShape {
 
 // Loader: stage rows first_row .. first_row+nrows-1 (clamped to [0,T)) x this block's column block of
 // `src` into `dst` (row pitch CB_BYTES). (row, piece) pairs are dealt round-robin to the loader waves.
-template <typename SH>
+// One direct global->LDS load of 16 bytes per lane; `once` picks the cache policy of rows no other tile reads.
+template <int ONCE_AUX>
+__device__ __forceinline__ void load_to_lds(rsrc_t rs, char* d, int voff, int so, bool once) {
+    if (kLoadAux != ONCE_AUX && once) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, voff, so, 0, ONCE_AUX);
+    else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, voff, so, 0, kLoadAux);
+}
+
+// `edge` = number of staged rows at either end that the neighbouring tile stages too (2P for a tile with its
+// K-1 halo rows, 0 for a tile without halo).
+template <typename SH, int ONCE_AUX>
 __device__ __forceinline__ void stage_rows(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
-                                           size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw, int lane) {
+                                           size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw, int lane,
+                                           int edge) {
     const int rb = first_row > 0 ? first_row : 0;
     const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
     const int rowb = (int)row_bytes;
@@ -133,8 +143,7 @@ __device__ __forceinline__ void stage_rows(const void* __restrict__ src, char* d
         const int p = pair % SH::NPIECE;
         const int so = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0 + p * 1024;
         char* d = dst + j * SH::CB_BYTES + p * 1024;
-        if (p * 1024 + voff < valid_bytes)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, voff, so, 0, 0);
+        if (p * 1024 + voff < valid_bytes) load_to_lds<ONCE_AUX>(rs, d, voff, so, j >= edge && j < nrows - edge);
     }
 }
 
@@ -143,10 +152,10 @@ __device__ __forceinline__ void stage_rows(const void* __restrict__ src, char* d
 // "all but the newest CNT loads have landed" is a compile-time s_waitcnt. Column blocks that are not
 // a whole number of 1 KiB pieces mask the lanes past the end instead (their LDS slots belong to the
 // next row); a piece with no lane left is then skipped, which only the plain "wait for all" tolerates.
-template <typename SH, int CNT>
+template <typename SH, int CNT, int ONCE_AUX>
 __device__ __forceinline__ void stage_rows_fixed(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
                                                  size_t row_bytes, int col_byte0, int valid_bytes, int lw, int nlw,
-                                                 int lane) {
+                                                 int lane, int edge) {
     const int rb = first_row > 0 ? first_row : 0;
     const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
     const int rowb = (int)row_bytes;
@@ -162,7 +171,7 @@ __device__ __forceinline__ void stage_rows_fixed(const void* __restrict__ src, c
         boff = inside ? boff : valid_bytes - 16;
         const int so = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0;
         char* d = dst + j * SH::CB_BYTES + p * 1024;
-        if (SH::WHOLE_PIECES || inside) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void*)d, 16, boff, so, 0, 0);
+        if (SH::WHOLE_PIECES || inside) load_to_lds<ONCE_AUX>(rs, d, boff, so, j >= edge && j < nrows - edge);
     }
 }
 
@@ -294,11 +303,11 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     const int ntl = (g.ntiles + g.nbt - 1) / g.nbt;        // rounds of the grid, the same for every block
     const size_t in_row_bytes = GATED ? 2 * row_bytes : row_bytes;   // pitch of x (z when gated)
     auto stage_tile = [&](char* buf, int first_row) {
-        stage_rows_fixed<SH, CNT>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
-                                  NWL, lane);
+        stage_rows_fixed<SH, CNT, kLoadAuxOnceFwd>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
+                                  NWL, lane, 2 * P);
         if constexpr (GATED)
-            stage_rows_fixed<SH, CNT>(x, buf + SH::TILE_BYTES, first_row, SH::NROWS, T, in_row_bytes, rowb + col_byte0,
-                                      valid_bytes, wv - SH::NWC, NWL, lane);
+            stage_rows_fixed<SH, CNT, kLoadAuxOnceFwd>(x, buf + SH::TILE_BYTES, first_row, SH::NROWS, T, in_row_bytes, rowb + col_byte0,
+                                      valid_bytes, wv - SH::NWC, NWL, lane, 2 * P);
     };
 
     // compute-wave coordinates (meaningless but harmless for loader waves)
@@ -546,18 +555,18 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 
     const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;    // pitch of x and dx (z and dz when gated)
     auto stage_x = [&](char* buf, int t0, int l, int nl) {
-        stage_rows<SH>(x, buf + SH::TILE_BYTES, t0, R, T, x_row_bytes, col_byte0, valid_bytes, l, nl, lane);
+        stage_rows<SH, kLoadAuxOnceBwdX>(x, buf + SH::TILE_BYTES, t0, R, T, x_row_bytes, col_byte0, valid_bytes, l, nl, lane, 0);
         if constexpr (GATED)
-            stage_rows<SH>(x, buf + SH::TILE_BYTES + XT_BYTES, t0, R, T, x_row_bytes, rowb + col_byte0, valid_bytes, l, nl,
-                           lane);
+            stage_rows<SH, kLoadAuxOnceBwdX>(x, buf + SH::TILE_BYTES + XT_BYTES, t0, R, T, x_row_bytes, rowb + col_byte0, valid_bytes, l, nl,
+                           lane, 0);
     };
     auto stage_both = [&](char* buf, int t0) {
         // with two or more loader waves, even ones take the dy tile and odd ones the x tile(s)
         if constexpr (WDW && NWL >= 2) {
             if (lw & 1) stage_x(buf, t0, lw >> 1, NWL / 2);
-            else        stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane);
+            else        stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane, 2 * P);
         } else {
-            stage_rows<SH>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane);
+            stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane, 2 * P);
             if constexpr (WDW) stage_x(buf, t0, lw, NWL);
         }
     };
