@@ -50,8 +50,8 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
 # profiles/bench_cfg3_hbm_traffic.md): keyed by (workload name, kernel). Counters cannot be read from
 # inside this process, so a workload without an entry reports traffic = null and says why.
 MEASURED_TRAFFIC = {
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 545113439,    # 1.015 x algorithmic
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 824575990,   # 1.024 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544046769,    # 1.013 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816835497,   # 1.014 x algorithmic
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
