@@ -199,7 +199,7 @@ int make_lds_plan(bool bwd, bool bf16, long long T, int C, int K, const nplm_dwc
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    p.sh = gated ? lds_gated_shape(bwd, bf16, lds_gated_narrow((long long)C * E), K) : lds_shape_for(bwd, bf16, K, (long long)C * E);
+    p.sh = gated ? lds_gated_shape(bwd, bf16, lds_gated_narrow((long long)C * E, K), K) : lds_shape_for(bwd, bf16, K, (long long)C * E);
     if (tune->vec > 0) p.sh.vec = tune->vec;
     if (tune->unroll > 0) p.sh.rw = tune->unroll;
     if (tune->bt > 0) p.sh.nrg = tune->bt;
@@ -307,11 +307,21 @@ hipError_t fill_zero(float* p, long long n, hipStream_t s) {
 
 // launch flags of the kernels (W_BF16 | W_RESIDUAL) from the ABI's weight dtype and flags
 // Shapes the gated (z = [u | g]) kernels are built for.
-bool gated_supported(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+bool gated_supported(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     const int E = bf16 ? 2 : 4;
-    if (!lds_gated_kernel_size(K) || T < 1) return false;
+    if (!lds_gated_kernel_size(K, bwd) || T < 1) return false;
     if (((long long)C * E) % 16 || align_bits % 16) return false;
     return (long long)C * E >= 1024;
+}
+
+// Long gated backward (K = 15, 31): the sliding-window kernel with one channel per lane; same shapes as the gated forward.
+bool long_gated_bwd_supported(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    return long_gated_kernel_size(K) && gated_supported(false, bf16, T, C, K, align_bits);
+}
+int make_long_gated_plan(bool bf16, long long T, int C, int K, Plan* out) {
+    nplm_dwconv_tuning t{};
+    t.vec = 1;
+    return make_plan(true, bf16, T, C, K, 0, &t, out);
 }
 
 int kernel_w_flags(int32_t w_dtype, uint32_t flags) {
@@ -526,16 +536,18 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
-    if (!gated_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)y)) return -NPLM_DWCONV_EUNSUPPORTED;
+    if (!gated_supported(false, bf16, T, C, K, (uintptr_t)z | (uintptr_t)y)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp;
     rc = make_lds_plan(false, bf16, T, C, K, nullptr, &lp, true);
     if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
     const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
-    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4));
+    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4), K);
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.ncb * lp.nbt);
     hipStream_t s = (hipStream_t)stream;
     switch (K) {
+        case 15: return (int)launch_fwd_lds_gated_k15(bf16, narrow, la, g, grid, s);
+        case 31: return (int)launch_fwd_lds_gated_k31(bf16, narrow, la, g, grid, s);
         case 3: return (int)launch_fwd_lds_gated_k3(bf16, narrow, la, g, grid, s);
         case 5: return (int)launch_fwd_lds_gated_k5(bf16, narrow, la, g, grid, s);
         case 7: return (int)launch_fwd_lds_gated_k7(bf16, narrow, la, g, grid, s);
@@ -547,7 +559,13 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
 size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
-    if (!gated_supported(bf16, T, C, K, 0)) return 0;
+    if (long_gated_bwd_supported(bf16, T, C, K, 0)) {
+        Plan p;
+        if (make_long_gated_plan(bf16, T, C, K, &p)) return 0;
+        const size_t bytes = (size_t)p.nbt * (K + 1) * C * sizeof(float);
+        return (bytes + 255) & ~(size_t)255;
+    }
+    if (!gated_supported(true, bf16, T, C, K, 0)) return 0;
     LdsPlan lp;
     if (make_lds_plan(true, bf16, T, C, K, nullptr, &lp, true)) return 0;
     const size_t bytes = (size_t)lp.nbt * (K + 1) * C * sizeof(float);
@@ -571,7 +589,26 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
-    if (!gated_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
+    if (long_gated_bwd_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
+        Plan p;
+        rc = make_long_gated_plan(bf16, T, C, K, &p);
+        if (rc) return rc;
+        const size_t slab = (size_t)(K + 1) * C * sizeof(float);
+        if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab * (size_t)p.nbt) return -NPLM_DWCONV_EWORKSPACE;
+        float* part = reinterpret_cast<float*>(workspace);
+        const ConvPtrs a{z, dy, cu, w, nullptr, dz, part};
+        const Geo g = make_geo(p, T, C, S, kernel_w_flags(w_dtype, flags));
+        const dim3 grid(p.ncb * p.nbt), block(p.bw * p.bt * 64);
+        const size_t shmem = (size_t)p.bw * p.bt * p.vec * 64 * sizeof(float);
+        hipError_t e = K == 15 ? launch_bwd_gated_k15(bf16, p.unroll, p.maxt, a, g, grid, block, shmem, s)
+                               : launch_bwd_gated_k31(bf16, p.unroll, p.maxt, a, g, grid, block, shmem, s);
+        if (e != hipSuccess) return (int)e;
+        const long long n_out = (long long)(K + 1) * C;
+        hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                           (const float*)part, p.nbt, C, K, dw, db);
+        return (int)hipGetLastError();
+    }
+    if (!gated_supported(true, bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp;
     rc = make_lds_plan(true, bf16, T, C, K, nullptr, &lp, true);
     if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
@@ -580,7 +617,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         return -NPLM_DWCONV_EWORKSPACE;
     float* part = reinterpret_cast<float*>(workspace);
     const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
-    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4));
+    const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4), K);
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.ncb * lp.nbt);
     hipError_t e = hipErrorInvalidConfiguration;

@@ -32,6 +32,13 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
     return __builtin_bit_cast(uint16_t, r);
 }
 
+// SwiGLU gate of the reference MLP (modeling.py:300-302: F.silu(gate) * x_proj), in fp32:
+// sig = 1 / (1 + 2^(-g log2 e)); h = u * g * sig. Also what the backward needs of it.
+__device__ __forceinline__ float sigmoid_f32(float g) {
+    return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g));
+}
+__device__ __forceinline__ float gate_mul(float u, float g) { return u * g * sigmoid_f32(g); }
+
 // ---------------------------------------------------------------------------------------------
 // Buffer addressing. Row slices are moved with MUBUF instructions: address = descriptor base +
 // scalar byte offset (the row, wave-uniform) + per-lane byte offset (the channel slice, constant for

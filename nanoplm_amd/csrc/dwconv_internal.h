@@ -103,6 +103,14 @@ NPLM_DECLARE_LDS_GATED_K(5)
 NPLM_DECLARE_LDS_GATED_K(7)
 NPLM_DECLARE_LDS_GATED_K(9)
 #undef NPLM_DECLARE_LDS_GATED_K
+// long gated kernels: sliding-window fused backward with one channel per lane,
+hipError_t launch_bwd_gated_k15(bool bf16, int unroll, int maxt, const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block,
+                                size_t shmem, hipStream_t s);
+hipError_t launch_bwd_gated_k31(bool bf16, int unroll, int maxt, const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block,
+                                size_t shmem, hipStream_t s);
+// and LDS-staged forward with the gate formed in LDS by the loader waves
+hipError_t launch_fwd_lds_gated_k15(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
 NPLM_DECLARE_LDS_K(7)
@@ -192,14 +200,19 @@ constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_by
 // Rows that are a multiple of 768 bytes but not of 1 KiB (C = 1152 in bf16, the reference's default
 // intermediate width) take 768-byte column blocks: 3 wave-columns; forward 2 row groups of 16 rows, backward
 // 3 row groups of 8 rows with 3 loader waves (12 waves: the registers of the gated backward need it).
-constexpr bool lds_gated_narrow(long long row_bytes) { return row_bytes % 768 == 0 && row_bytes % 1024 != 0; }
+// Long gated forward (K = 15, 31): 512-byte column blocks (2 wave-columns x 4 bytes per lane), 4 row groups of 8 rows,
+// 4 loader waves that also form h = u * silu(g) in LDS once per staged element (gate_prepass); two (u, g) tile
+// pairs of 32 + K-1 rows = 124 KiB at K = 31.
+constexpr bool lds_gated_narrow(long long row_bytes, int K = 7) { return K <= 9 && row_bytes % 768 == 0 && row_bytes % 1024 != 0; }
 constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16, bool narrow = false, int K = 7) {
+    if (K >= 15) return LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 4, 2, 8, 2};
     // narrow: one shape for every K <= 9 (at K = 9 in bf16 the backward spills 5 registers; a variant with fewer
     // waves and no spill measured slower: 440 against 334 us at T=131072, C=1152)
     if (narrow) return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 3, 3, 3, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 3, 4, 2};
     return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, (bwd && K == 3) ? 3 : 2, 4, 4, 2};
 }
-constexpr bool lds_gated_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+constexpr bool lds_gated_kernel_size(int K, bool bwd) { return K == 3 || K == 5 || K == 7 || K == 9 || (!bwd && (K == 15 || K == 31)); }
+constexpr bool long_gated_kernel_size(int K) { return K == 15 || K == 31; }   // backward: sliding-window kernel, gated
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)bwd; (void)K; (void)vec;
     return 256;

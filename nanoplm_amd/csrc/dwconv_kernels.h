@@ -259,7 +259,10 @@ dwconv_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, co
 // waves of a block that share a wave-column are summed through LDS in fixed order (token slot
 // 0,1,2,...), and the block writes one slab partial[tb][k][c]. No atomics.
 // WDX / WDW select the outputs at compile time (dx only, dw/db only, or both).
-template <bool BF16, int K, int VEC, int U, int MAXT, bool WDX, bool WDW>
+// GATED: x is z = [u | g] of shape [T, 2C] (the SwiGLU MLP's Wi output, modeling.py:300-302), the conv ran over
+// h = u * silu(g), and dx is dz [T, 2C] = [dh * silu(g) | dh * u * sig(g) * (1 + g * (1 - sig(g)))] with dh the
+// conv's input gradient; h (for dw) and the two gate factors are formed once per element from the centre rows.
+template <bool BF16, int K, int VEC, int U, int MAXT, bool WDX, bool WDW, bool GATED = false>
 __global__ void __launch_bounds__(MAXT)
 dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                   const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const Geo g) {
@@ -267,6 +270,7 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
     constexpr int E = BF16 ? 2 : 4;
     using Row = RowVec<BF16, VEC>;
     using RG = Ring<K, U>;
+    static_assert(!GATED || (WDX && WDW), "the gated backward always produces dz, dw and db");
     extern __shared__ float red[];   // [nwaves][VEC][64]
 
     const int lane = (int)(threadIdx.x & 63);
@@ -286,6 +290,8 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
     const int lane_off = c0 * E;
     const size_t row_bytes = (size_t)g.C * E;
     const int rowb = (int)row_bytes;
+    const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;    // pitch of x and dx (z and dz when gated)
+    const int xrowb = (int)x_row_bytes;
     const int T = g.T, S = g.S, R = g.R;
 
     float wr[VEC][K];
@@ -308,8 +314,8 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
             const int t1 = (t0 + R < T) ? t0 + R : T;
             const int rb = (t0 - P > 0) ? t0 - P : 0;
             const rsrc_t rg = rows_rsrc(dy, rb, T, row_bytes);   // dy rows from rb (window with halo)
-            const rsrc_t rx = rows_rsrc(x, t0, T, row_bytes);    // x rows from t0 (centre rows only)
-            const rsrc_t ro = rows_rsrc(dx, t0, T, row_bytes);
+            const rsrc_t rx = rows_rsrc(x, t0, T, x_row_bytes);  // x rows from t0 (centre rows only)
+            const rsrc_t ro = rows_rsrc(dx, t0, T, x_row_bytes);
 
             float gw[RG::RING][VEC];   // slot(ph, j) holds dy row tc - P + j
 #pragma unroll
@@ -318,11 +324,12 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                 r.bload(rg, lane_off, (clamp_row(t0 - P + j, T) - rb) * rowb);
                 r.to_f32(gw[RG::slot(0, j)]);
             }
-            Row nx[WDW ? U : 1], ng[U];
+            Row nx[WDW ? U : 1], nxg[GATED ? U : 1], ng[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 ng[u].bload(rg, lane_off, (clamp_row(t0 + P + u, T) - rb) * rowb);
-                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(t0 + u, T) - t0) * rowb);
+                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(t0 + u, T) - t0) * xrowb);
+                if constexpr (GATED) nxg[u].bload(rx, lane_off + rowb, (clamp_row(t0 + u, T) - t0) * xrowb);
             }
             sc.locate(cu, S, T, t0, sc.seq);
 
@@ -331,21 +338,35 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                 static_for<RG::NPH>([&](auto ph_c) {
                     constexpr int ph = decltype(ph_c)::value;
                     if (tc < t1) {
-                        float xc[WDW ? U : 1][VEC];   // x rows tc .. tc+U-1
+                        float xc[WDW ? U : 1][VEC];   // x rows tc .. tc+U-1 (h rows when gated)
+                        // gated: gs = g * sig(g) (h = u * gs, du = dh * gs), gd = u * sig(g) * (1 + g * (1 - sig(g))) (dg = dh * gd)
+                        float gs[GATED ? U : 1][VEC], gd[GATED ? U : 1][VEC];
 #pragma unroll
                         for (int u = 0; u < U; ++u) {
                             ng[u].to_f32(gw[RG::slot(ph, K - 1 + u)]);
                             if constexpr (WDW) nx[u].to_f32(xc[u]);
+                            if constexpr (GATED) {
+                                float gg[VEC];
+                                nxg[u].to_f32(gg);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) {
+                                    const float sg = sigmoid_f32(gg[v]);
+                                    gs[u][v] = gg[v] * sg;
+                                    gd[u][v] = xc[u][v] * sg * (1.f + gg[v] * (1.f - sg));
+                                    xc[u][v] *= gs[u][v];
+                                }
+                            }
                         }
                         if (tc + U < t1) {
 #pragma unroll
                             for (int u = 0; u < U; ++u) {
                                 ng[u].bload(rg, lane_off, (clamp_row(tc + U + P + u, T) - rb) * rowb);
-                                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(tc + U + u, T) - t0) * rowb);
+                                if constexpr (WDW) nx[u].bload(rx, lane_off, (clamp_row(tc + U + u, T) - t0) * xrowb);
+                                if constexpr (GATED) nxg[u].bload(rx, lane_off + rowb, (clamp_row(tc + U + u, T) - t0) * xrowb);
                             }
                         }
                         sc.advance(cu, S, T, tc);
-                        Row o[WDX ? U : 1];
+                        Row o[WDX ? U : 1], og[GATED ? U : 1];
                         if (tc - P >= sc.cs && tc + U - 1 + P < sc.ce && tc + U <= t1) {
 #pragma unroll
                             for (int u = 0; u < U; ++u) {
@@ -363,12 +384,23 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                         if constexpr (WDX) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
                                         if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - m]);
                                     }
-                                if constexpr (WDX) o[u].from_f32(acc);
+                                if constexpr (GATED) {
+                                    float du[VEC], dg[VEC];
+#pragma unroll
+                                    for (int v = 0; v < VEC; ++v) { du[v] = acc[v] * gs[u][v]; dg[v] = acc[v] * gd[u][v]; }
+                                    o[u].from_f32(du);
+                                    og[u].from_f32(dg);
+                                } else if constexpr (WDX) {
+                                    o[u].from_f32(acc);
+                                }
                             }
                             if constexpr (WDX) {
                                 if (active) {
 #pragma unroll
-                                    for (int u = 0; u < U; ++u) o[u].bstore(ro, lane_off, (tc + u - t0) * rowb);
+                                    for (int u = 0; u < U; ++u) {
+                                        o[u].bstore(ro, lane_off, (tc + u - t0) * xrowb);
+                                        if constexpr (GATED) og[u].bstore(ro, lane_off + rowb, (tc + u - t0) * xrowb);
+                                    }
                                 }
                             }
                         } else {
@@ -394,7 +426,17 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                             if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - m]);
                                         }
                                     }
-                                    if constexpr (WDX) {
+                                    if constexpr (GATED) {
+                                        float du[VEC], dg[VEC];
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v) { du[v] = acc[v] * gs[u][v]; dg[v] = acc[v] * gd[u][v]; }
+                                        o[u].from_f32(du);
+                                        og[u].from_f32(dg);
+                                        if (active) {
+                                            o[u].bstore(ro, lane_off, (t - t0) * xrowb);
+                                            og[u].bstore(ro, lane_off + rowb, (t - t0) * xrowb);
+                                        }
+                                    } else if constexpr (WDX) {
                                         o[u].from_f32(acc);
                                         if (active) o[u].bstore(ro, lane_off, (t - t0) * rowb);
                                     }

@@ -189,13 +189,6 @@ __device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
     r.to_f32(f);
 }
 
-// SwiGLU gate of the reference MLP (modeling.py:300-302: F.silu(gate) * x_proj), in fp32:
-// sig = 1 / (1 + 2^(-g log2 e)); h = u * g * sig. Also what the backward needs of it.
-__device__ __forceinline__ float sigmoid_f32(float g) {
-    return __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g));
-}
-__device__ __forceinline__ float gate_mul(float u, float g) { return u * g * sigmoid_f32(g); }
-
 // One lane's slice of a gated input row out of LDS: h[v] = u[v] * silu(g[v]).
 template <bool BF16, int VEC>
 __device__ __forceinline__ void lds_read_gated_row(const char* pu, const char* pg, float (&h)[VEC]) {
@@ -261,6 +254,52 @@ __device__ __forceinline__ void wave_tap_masks(SeqCursor sc, int nce, const int3
     }
 }
 
+// Long gated kernels (K >= 15): a wave reads RW+K-1 staged rows for RW output rows, so a gate evaluated as rows are
+// read would be evaluated (RW+K-1)/RW times per element. Instead the loader waves, once a tile has landed, turn
+// its u and g rows into h = u * silu(g) in place, in fp32: a lane takes EPL adjacent elements of a row (the same
+// bytes of the u row and of the g row) and leaves the first half of its h values where its u elements were and
+// the second half where its g elements were (fp32 activations: all of them where u was). The compute waves then
+// read fp32 h and do no gate arithmetic (and no bf16 unpacking) at all.
+template <typename SH, bool BF16>
+__device__ __forceinline__ void gate_prepass(char* buf, int lw, int nlw, int lane) {
+    constexpr int EPL = SH::CB_CH / 64;
+    static_assert(EPL == 2 || EPL == 4 || EPL == 8, "elements per lane and row");
+    for (int j = lw; j < SH::NROWS; j += nlw) {
+        char* pu = buf + j * SH::CB_BYTES + lane * EPL * SH::E;
+        char* pg = pu + SH::TILE_BYTES;
+        float u[EPL], g[EPL], h[EPL];
+        lds_read_row<BF16, EPL>(pu, u);
+        lds_read_row<BF16, EPL>(pg, g);
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) h[i] = gate_mul(u[i], g[i]);
+        if constexpr (BF16) {
+            RowVec<false, EPL / 2> lo, hi;
+#pragma unroll
+            for (int i = 0; i < EPL / 2; ++i) { lo.v[i] = h[i]; hi.v[i] = h[EPL / 2 + i]; }
+            lo.store(pu);
+            hi.store(pg);
+        } else {
+            RowVec<false, EPL> o;
+#pragma unroll
+            for (int i = 0; i < EPL; ++i) o.v[i] = h[i];
+            o.store(pu);
+        }
+    }
+}
+// Byte offset inside a staged row of the fp32 h values of channels lc .. lc+VEC-1 of the column block.
+template <typename SH, bool BF16, int VEC>
+__device__ __forceinline__ int pregated_offset(int lc) {
+    constexpr int EPL = SH::CB_CH / 64;
+    if constexpr (BF16) {
+        static_assert(VEC <= EPL / 2, "a lane's channels lie in one half of a pre-pass lane's elements");
+        const int l = lc / EPL, r = lc % EPL;
+        const bool second = r >= EPL / 2;
+        return (second ? SH::TILE_BYTES : 0) + l * EPL * 2 + (r - (second ? EPL / 2 : 0)) * 4;
+    } else {
+        return lc * 4;
+    }
+}
+
 // =============================================================================================
 // Forward
 // =============================================================================================
@@ -282,6 +321,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     static_assert(NBUF == 2 || NBUF == 3, "two or three tile buffers");
     static_assert(NBUF == 2 || SH::WHOLE_PIECES, "three buffers count loads in flight: whole 1 KiB pieces only");
     static_assert(!GATED || NBUF == 2, "the gated forward is double-buffered");
+    constexpr bool PREGATE = GATED && K >= 15;   // the loader waves form h in LDS (see gate_prepass)
     // Where LDS has 32 bytes to spare per row group, the loader waves (idle while their loads are in
     // flight) also run the boundary lookup for the next tile and leave the result in a mailbox behind
     // the tile buffers; the compute waves, whose stores make them as memory-bound as the loaders, then
@@ -351,6 +391,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
         } else {
             wait_vmem_all();
         }
+        if constexpr (PREGATE) gate_prepass<SH, BF16>(lds_raw, wv - SH::NWC, NWL, lane);
     } else {
         load_weights<VEC, K>(w, g.w_flags, c0, wr);
         if (b) {
@@ -384,6 +425,9 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
             }
             if (it + 1 < ntl) post_bounds((it + 1) & 1, lds_tile_row0(g, it + 1, qn, R));
             if (NBUF == 3 && rn < T) wait_vmem_but<CNT>(); else wait_vmem_all();
+            if constexpr (PREGATE) {
+                if (rn < T) gate_prepass<SH, BF16>(lds_raw + ((bcur + 1) % NBUF) * BUF_BYTES, wv - SH::NWC, NWL, lane);
+            }
         } else {
             const int tf = t0 + rg * RW;
             if (tf < T) {
@@ -401,12 +445,13 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                 for (int u = 0; u < RW; ++u)
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[u][v] = bias[v];
-                const char* lp = cur + (rg * RW) * SH::CB_BYTES + lc0 * E;
+                const char* lp = cur + (rg * RW) * SH::CB_BYTES + (PREGATE ? pregated_offset<SH, BF16, VEC>(lc0) : lc0 * E);
                 if (interior) {
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float xr[VEC];
-                        if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
+                        if constexpr (PREGATE) lds_read_row<false, VEC>(lp + j * SH::CB_BYTES, xr);
+                        else if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
                         else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
@@ -443,7 +488,8 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         for (int j = 0; j < RW + K - 1; ++j) {
                             if (j >= jlo && j < jhi) {
                                 float xr[VEC];
-                                if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
+                                if constexpr (PREGATE) lds_read_row<false, VEC>(lp + j * SH::CB_BYTES, xr);
+                                else if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
                                 else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
 #pragma unroll
                                 for (int u = 0; u < RW; ++u) {

@@ -46,6 +46,34 @@ def test_gated_kernel_sizes_and_widths(K, dt, C):
     _check(*_case(LENS_MIX, C, K, dt, dt, seed=K + C), f"gated K={K} C={C} {dt}")
 
 
+LENS_LONG = LENS_MIX + [40, 33, 31, 30, 29, 16, 15, 14, 0, 1, 1, 700]
+
+
+@pytest.mark.parametrize("K", [15, 31])
+@pytest.mark.parametrize("dt,wdt,C", [(torch.bfloat16, torch.bfloat16, 1024), (torch.bfloat16, torch.float32, 2048),
+                                       (torch.bfloat16, torch.bfloat16, 520), (torch.float32, torch.float32, 256),
+                                       (torch.float32, torch.float32, 776), (torch.bfloat16, torch.bfloat16, 1152)])
+def test_long_gated_kernel_sizes_and_widths(K, dt, wdt, C):
+    """K = 15 and 31 (the intermediate-width configuration is C = 2048, K = 31): the forward forms the gate product in
+    LDS once per staged element, the backward is the sliding-window kernel with the gate on its centre rows."""
+    print(f"[case] long gated K={K} C={C} {dt} w {wdt}", flush=True)
+    _check(*_case(LENS_LONG, C, K, dt, wdt, seed=K + C), f"gated K={K} C={C} {dt}")
+    _check(*_case(LENS_LONG[::-1], C, K, dt, wdt, seed=K + C + 1), f"gated residual K={K} C={C} {dt}", residual=True)
+
+
+def test_long_gated_is_deterministic_and_takes_the_boundary_stress_mix():
+    wl = make_workload(5, T=20011, C=1024, with_dy=True)        # lengths of 1..8 mixed with 400..512, odd T
+    g = torch.Generator().manual_seed(19)
+    z = torch.randn(wl.T, 2048, generator=g).bfloat16()
+    w = (torch.randn(1024, 31, generator=g) * 31 ** -0.5).bfloat16()
+    _check(z, wl.cu_seqlens, w, wl.bias, wl.dy, "long gated boundary stress")
+    zd, cud, wd, dyd = z.to(DEV), wl.cu_seqlens.to(DEV), w.to(DEV), wl.dy.to(DEV)
+    a = npa.gated_dwconv_bwd(zd, dyd, cud, wd)
+    b = npa.gated_dwconv_bwd(zd, dyd, cud, wd)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
+    assert torch.equal(npa.gated_dwconv_fwd(zd, cud, wd, None), npa.gated_dwconv_fwd(zd, cud, wd, None))
+
+
 def test_gated_intermediate_width_with_fp32_weights_and_residual():
     _check(*_case(LENS_MIX, 2048, 7, torch.bfloat16, torch.float32, seed=4), "gated C=2048 bf16/fp32")
     _check(*_case(LENS_MIX, 1024, 7, torch.bfloat16, torch.bfloat16, seed=6), "gated residual", residual=True)
