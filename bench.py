@@ -47,11 +47,17 @@ HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and
 # scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
-# profiles/bench_cfg3_hbm_traffic.md): keyed by (workload name, kernel). Counters cannot be read from
-# inside this process, so a workload without an entry reports traffic = null and says why.
+# profiles/bench_cfg3_hbm_traffic.md and profiles/bench_cfg2_cfg4_cfg5_hbm_traffic.md): keyed by
+# (workload name, kernel). Counters cannot be read from inside this process, so a workload or variant
+# without an entry (configuration 1, --gated, --residual) reports traffic = null and says why.
 MEASURED_TRAFFIC = {
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544046769,    # 1.013 x algorithmic
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816835497,   # 1.014 x algorithmic
+    ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136282529,                       # 1.015 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544046769,                   # 1.013 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816835497,                  # 1.014 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1258207411,       # 1.172 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1691043683,      # 1.050 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272216838,    # 1.014 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410635307,   # 1.020 x
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
