@@ -192,24 +192,33 @@ constexpr LdsShapeSel lds_shape_for(bool bwd, bool bf16, int K, long long row_by
                                             : lds_default_shape(bwd, bf16, K);
 }
 // Gated kernels (z = [u | g] input): 1 KiB column blocks, so that a u tile and a g tile fit where the plain
-// kernels hold one x tile: 4 wave-columns x 4 bytes per lane, 2 row groups, 4 loader waves. The gate
-// costs two transcendentals per element read, so the forward takes 32-row tiles (16 rows per wave: the
-// K-1 halo rows it re-gates weigh less; 2 x 2 x 38 KiB = 152 KiB of LDS at K = 7), the backward 16-row
-// tiles (2 x (22 + 16 + 16) KiB = 108 KiB). Taller backward tiles would stream better (K = 3, whose registers
-// allow a third row group: 297 -> 254 us at T=131072, C=1024) but spill from K = 5 on (K = 7: 295 -> 328 us).
+// kernels hold one x tile: 4 wave-columns x 4 bytes per lane, 4 loader waves. The gate costs two transcendentals
+// per element read, so the forward takes 32-row tiles of 2 row groups (16 rows per wave: the K-1 halo rows it
+// re-gates weigh less; 2 x 2 x 38 KiB = 152 KiB of LDS at K = 7). The backward evaluates the gate on its x rows only
+// (no halo) and its vector-ALU work (about 40 instructions per element) is what it has to hide behind the stream:
+// 3 row groups, i.e. 12 compute waves, with as many rows per wave as 128 registers hold. Measured at T=131072,
+// C=1024, bf16 against 2 row groups of 8 rows (backward + finalize, us): K = 5: 289 -> 240 with 7 rows per wave
+// (8 rows: 257, 6: 277); K = 7: 294 -> 250 with 6 rows (7: 266, 8: 295, 5: 295); K = 9: 296 -> 272 with 5 rows (6: 281,
+// 7: 296). The few registers these shapes spill (8 at K = 7, 21 at K = 9) cost less than the narrower tiles save.
 // Rows that are a multiple of 768 bytes but not of 1 KiB (C = 1152 in bf16, the reference's default
-// intermediate width) take 768-byte column blocks: 3 wave-columns; forward 2 row groups of 16 rows, backward
-// 3 row groups of 8 rows with 3 loader waves (12 waves: the registers of the gated backward need it).
+// intermediate width) take 768-byte column blocks: 3 wave-columns; forward 2 row groups of 16 rows; backward
+// 4 row groups (12 compute + 4 loader waves) of 8 rows (bf16: 6 at K = 7, 5 at K = 9). Measured at T=131072,
+// C=1152, bf16 against 3 row groups of 8 rows with 3 loader waves (us): K = 3: 392 -> 292, 5: 383 -> 295, 7: 400 -> 292,
+// 9: 350 -> 299.
 // Long gated forward (K = 15, 31): 512-byte column blocks (2 wave-columns x 4 bytes per lane), 4 row groups of 8 rows,
-// 4 loader waves that also form h = u * silu(g) in LDS once per staged element (gate_prepass); two (u, g) tile
-// pairs of 32 + K-1 rows = 124 KiB at K = 31.
+// 8 loader waves that also form h = u * silu(g) in LDS once per staged element (gate_prepass; with 4 loader waves the
+// pre-pass is the longer half of a tile: 745 against 599 us at T=131072, C=2048, K=31); two (u, g) tile pairs of
+// 32 + K-1 rows = 124 KiB at K = 31.
 constexpr bool lds_gated_narrow(long long row_bytes, int K = 7) { return K <= 9 && row_bytes % 768 == 0 && row_bytes % 1024 != 0; }
 constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16, bool narrow = false, int K = 7) {
     if (K >= 15) return LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 4, 2, 8, 2};
-    // narrow: one shape for every K <= 9 (at K = 9 in bf16 the backward spills 5 registers; a variant with fewer
-    // waves and no spill measured slower: 440 against 334 us at T=131072, C=1152)
-    if (narrow) return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 3, 3, 3, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 3, 4, 2};
-    return LdsShapeSel{bf16, bf16 ? 2 : 1, bwd ? 8 : 16, (bwd && K == 3) ? 3 : 2, 4, 4, 2};
+    if (narrow)
+        return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, bf16 ? (K <= 5 ? 8 : K <= 7 ? 6 : 5) : 8, 4, 3, 4, 2}
+                   : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 3, 4, 2};
+    // backward: 3 row groups (12 compute + 4 loader waves, 128 registers each); in bf16 the rows per wave shrink with K
+    // so that the two cached gate factors per element still fit: 8, 7, 6, 5 rows at K = 3, 5, 7, 9
+    if (bwd) return LdsShapeSel{bf16, bf16 ? 2 : 1, bf16 ? (K <= 3 ? 8 : K <= 5 ? 7 : K <= 7 ? 6 : 5) : 8, 3, 4, 4, 2};
+    return LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
 }
 constexpr bool lds_gated_kernel_size(int K, bool bwd) { return K == 3 || K == 5 || K == 7 || K == 9 || (!bwd && (K == 15 || K == 31)); }
 constexpr bool long_gated_kernel_size(int K) { return K == 15 || K == 31; }   // backward: sliding-window kernel, gated
