@@ -166,19 +166,20 @@ constexpr int kLdsDefaultCb = 1024;
 // Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block
 // widths cover the common cases (K <= 9):
 //   backward, 768 bytes (C = 768 and 1152 in bf16, the reference's default hidden and intermediate widths,
-//       modeling.py:42-43): 3 wave-columns x 4 bytes per lane, 3 row groups of 16 rows (48-row tiles, so that a
-//       tile in flight is still ~75 KiB per CU); 9 compute + 7 loader waves (3 at K = 9 in bf16, for the
-//       registers), two (dy, x) tile pairs (153 KiB).
+//       modeling.py:42-43): 3 wave-columns x 4 bytes per lane, 4 row groups of 12 rows (48-row tiles, so that a
+//       tile in flight is still ~75 KiB per CU); 12 compute + 4 loader waves, two (dy, x) tile pairs (153 KiB).
+//       (3 row groups of 16 rows with 7 loader waves, 3 at K = 9 in bf16: C=768 K=7 120 against 112 us, K=9 135
+//       against 112 us; C=1152 K=9 188 against 162 us.)
 //   backward, 1280 bytes (C = 640, 1280 in bf16): 5 wave-columns x 4 bytes per lane, 2 row groups of 12 rows,
 //       10 compute + 6 loader waves, 135 KiB.
 //   forward, 2 KiB for rows between 1280 and 2047 bytes (C = 640 .. 1023 in bf16), which fill one such block
 //       better than two of 1 KiB: 4 wave-columns x 8 bytes per lane, 2 row groups of 8 rows, 4 loader waves.
-// Measured at T=131072, K=7, bf16 (us, default blocks -> these): backward C=768 140 -> 124, C=1152 200 -> 175,
+// Measured at T=131072, K=7, bf16 (us, default blocks -> these): backward C=768 140 -> 112, C=1152 200 -> 159,
 // C=640 135 -> 106, C=1280 208 -> 193; forward C=768 83 -> 76. The forward gains nothing from 768-byte blocks
 // (C=1152: 113 against 115, C=2304 at T=65536: 119 against 110).
 constexpr LdsShapeSel lds_narrow_shape(bool bwd, bool bf16, int K, int cb_bytes) {
     if (!bwd) return LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 4, 2};          // 2048, forward
-    if (cb_bytes == 768) return LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 3, 3, (bf16 && K >= 9) ? 3 : 7, 2};
+    if (cb_bytes == 768) return LdsShapeSel{bf16, bf16 ? 2 : 1, 12, 4, 3, 4, 2};
     return LdsShapeSel{bf16, bf16 ? 2 : 1, 12, 2, 5, 6, 2};                  // 1280, backward
 }
 // 0 = the default column block, else 768 or 1280 (backward), 2048 (forward)
