@@ -158,7 +158,7 @@ int nplm_dwconv_bwd_static(const void* x, const void* dy, const int32_t* cu, con
  *   y  = conv(h; w, b), h = z[:, :C] * silu(z[:, C:])           (h is formed in fp32, never stored)
  *   dz = [dh * silu(gate) | dh * x_proj * silu'(gate)], dh = conv^T(dy; w); dw, db as for conv(h)
  * This saves writing h and reading it back (forward) and the separate elementwise backward (backward).
- * Built for K in {3,5,7,9}, C * elemsize a multiple of 16 bytes and at least 1 KiB, 16-byte aligned
+ * Built for K in {3,5,7,9,15,31}, C * elemsize a multiple of 16 bytes and at least 1 KiB, 16-byte aligned
  * z / y / dy / dz; anything else returns -NPLM_DWCONV_EUNSUPPORTED and launches nothing (callers then
  * compose the unfused ops). `flags` as for nplm_dwconv_fwd_ex (the residual applies to h).
  * nplm_dwconv_gated_bwd_workspace_bytes returns 0 for unsupported shapes.
