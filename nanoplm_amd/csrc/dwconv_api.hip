@@ -271,15 +271,56 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
     return hipErrorInvalidConfiguration;
 }
 
-// algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged.
+// ---- role-split LDS-staged backward at K = 31 (dwconv_lds_split_kernels.h) ---------------------------
+bool split_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    const int E = bf16 ? 2 : 4;
+    if (!lds_split_kernel_size(K) || T < 1) return false;
+    if (((long long)C * E) % 16 || align_bits % 16) return false;
+    const SplitShapeSel sh = lds_split_shape(bf16, K);
+    return (long long)C * E >= (long long)sh.ncw * 64 * sh.vec * E;
+}
+int make_split_plan(bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
+    LdsPlan p{};
+    nplm_dwconv_tuning z{};
+    if (!tune) tune = &z;
+    const int E = bf16 ? 2 : 4;
+    const SplitShapeSel sh = lds_split_shape(bf16, K);
+    const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
+    const long long row_bytes = (long long)C * E;
+    p.R = sh.rw * sh.nrg;
+    if ((long long)(p.R + K) * row_bytes + 2 * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
+    p.ncb = ceil_div(row_bytes, cb_bytes);
+    p.ntiles = ceil_div(T, p.R);
+    int nbt = tune->nbt > 0 ? tune->nbt : kNumCU / p.ncb;     // one block of 16 waves per CU
+    if (nbt < 1) nbt = 1;
+    if (nbt > p.ntiles) nbt = p.ntiles;
+    if (tune->nbt <= 0) {
+        const long long cap = (long long)(kSlabBudgetBytes / ((size_t)(K + 1) * C * sizeof(float)));
+        if (nbt > cap && cap >= 1) nbt = (int)cap;
+    }
+    p.nbt = nbt;
+    int G = tune->xcd_remap == 0 ? 8 : (tune->xcd_remap > 0 ? tune->xcd_remap : 0);
+    const long long nblocks = (long long)p.ncb * p.nbt;
+    if (G > 0 && !(nblocks % kNumXCD == 0 && (nblocks / kNumXCD) % G == 0 && p.nbt % G == 0)) G = 0;
+    p.xcd_group = G;
+    p.rot_step = nbt > 2 ? (int)((long long)nbt * 618 / 1000) | 1 : 0;
+    if (p.rot_step >= nbt) p.rot_step = nbt - 1;
+    *out = p;
+    return 0;
+}
+
+// algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged, 3 role-split LDS-staged.
 // Measured on MI355X at T=131072, C=1024, K=7, bf16: both passes are fastest LDS-staged (the chip
 // sweeps one compact window of rows with every load of a tile issued at once). At K=31 (ALU-bound)
-// the LDS-staged forward still wins by ~17 % (C=1024 and 2048) but the fused backward does not fit
-// its registers, so it stays with the sliding-window kernel, like everything the LDS kernels are not
-// built for (K = 15, other sizes, narrow or unaligned rows).
+// the LDS-staged forward still wins by ~17 % (C=1024 and 2048); one wave cannot hold the fused backward's
+// registers there, so the backward that produces every output takes the role-split kernel (13 - 15 % faster than
+// the sliding-window one at C=2048) and a backward asked for dx alone or dw/db alone the sliding-window kernel,
+// like everything the LDS kernels are not built for (K = 15 backward, other sizes, narrow or unaligned rows).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    if (tune && tune->algo == 3) return (bwd && split_eligible(bf16, T, C, K, align_bits)) ? 3 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 2) return lds_eligible(bf16, T, C, K, align_bits) ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
+    if (bwd && split_eligible(bf16, T, C, K, align_bits)) return 3;
     return lds_preferred(bwd, bf16, T, C, K, align_bits) ? 2 : 1;
 }
 
@@ -399,8 +440,34 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
 
-    const int algo = choose_algo(true, tune, bf16, T, C, K, bits);
+    int algo = choose_algo(true, tune, bf16, T, C, K, bits);
     if (algo < 0) return algo;
+    if (algo == 3 && !(dx && want_red)) {     // the role-split kernel is fused only: a partial request takes the others
+        if (tune && tune->algo == 3) return -NPLM_DWCONV_ETUNING;
+        algo = 1;
+    }
+    if (algo == 3) {
+        LdsPlan lp;
+        rc = make_split_plan(bf16, T, C, K, tune, &lp);
+        if (rc) return rc;
+        const size_t slab_bytes = (size_t)(K + 1) * C * sizeof(float);
+        if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab_bytes * (size_t)lp.nbt)
+            return -NPLM_DWCONV_EWORKSPACE;
+        float* part = reinterpret_cast<float*>(workspace);
+        const ConvPtrs la{x, dy, cu, w, nullptr, dx, part};
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, w_flags);
+        const dim3 grid(lp.ncb * lp.nbt);
+        hipError_t e = launch_bwd_split_k31(bf16, la, lg, grid, s);
+        if (e != hipSuccess) return (int)e;
+        if (tune && tune->mid_event) {
+            e = hipEventRecord((hipEvent_t)tune->mid_event, s);
+            if (e != hipSuccess) return (int)e;
+        }
+        const long long n_out = (long long)(K + 1) * C;
+        hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0,
+                           s, (const float*)part, lp.nbt, C, K, dw, db);
+        return (int)hipGetLastError();
+    }
     if (algo == 2) {
         LdsPlan lp;
         rc = make_lds_plan(true, bf16, T, C, K, tune, &lp);
@@ -681,6 +748,10 @@ size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t 
         LdsPlan lp;
         if (make_lds_plan(true, bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
     }
+    if (split_eligible(bf16, T, C, K, 0)) {
+        LdsPlan lp;
+        if (make_split_plan(bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
+    }
     const size_t bytes = (size_t)slabs * (K + 1) * C * sizeof(float);
     return (bytes + 255) & ~(size_t)255;
 }
@@ -690,6 +761,11 @@ int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const int algo = choose_algo(true, tune, bf16, T, C, K, 0);
     if (algo < 0) return 0;
+    if (algo == 3) {
+        LdsPlan lp;
+        if (make_split_plan(bf16, T, C, K, tune, &lp)) return 0;
+        return lp.nbt;
+    }
     if (algo == 2) {
         LdsPlan lp;
         if (make_lds_plan(true, bf16, T, C, K, tune, &lp)) return 0;

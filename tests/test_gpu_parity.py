@@ -362,10 +362,65 @@ def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
         y = npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=tf)
         try:
             dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=tf)
-        except RuntimeError:         # no LDS-staged backward at K = 15, 31
+        except RuntimeError:         # no single-role LDS-staged backward at K = 15, 31
             assert algo == 2 and K in (15, 31)
             dx = None
         outs.append((y, dx))
     assert torch.equal(outs[0][0], outs[1][0])
     if outs[1][1] is not None:
         assert torch.equal(outs[0][1], outs[1][1])
+    if K == 31:                      # the role-split LDS-staged backward rotates its tile slots the same way
+        dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+        assert torch.equal(dx, outs[0][1])
+
+
+# ---- role-split LDS-staged backward (K = 31) ---------------------------------------------------------
+LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 16, 17, 30, 31, 32, 33, 700, 1, 1, 1,
+              29, 0, 0, 45, 1200, 14]
+
+
+@pytest.mark.parametrize("C,dt", [(256, torch.bfloat16), (264, torch.bfloat16), (1024, torch.bfloat16),
+                                  (1152, torch.bfloat16), (2048, torch.bfloat16), (2056, torch.bfloat16),
+                                  (128, torch.float32), (388, torch.float32), (1024, torch.float32)])
+@pytest.mark.parametrize("nbt", [0, 1, 5])
+def test_role_split_backward_matches_the_sliding_window_kernel_and_the_oracle(C, dt, nbt):
+    """A fused K = 31 backward is served by a kernel whose waves are split into a dx role and a dw/db role over the
+    same LDS tiles. Sequences shorter than the 15-row halo, tile-edge lengths, empty sequences, partial column
+    blocks and one or a few blocks walking every tile: dx must equal the sliding-window kernel's bit for bit, and
+    dw/db the oracle's to the reduction tolerance."""
+    print(f"[case] C={C} {dt} nbt={nbt}", flush=True)
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, C, 31, dt, dt, seed=C + nbt)
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
+    xd, cud, wd, dyd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV)
+    dx1, dw1, db1 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=1))
+    dx3, dw3, db3 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    assert torch.equal(dx3, dx1)
+    assert_act_close(dx3, dx64, dt, "dx")
+    assert_red_close(dw3, dw64, "dw")
+    assert_red_close(db3, db64, "db")
+    torch.testing.assert_close(dw3, dw1, rtol=1e-5, atol=1e-3)
+    again = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    assert all(torch.equal(a, b_) for a, b_ in zip(again, (dx3, dw3, db3)))      # fixed summation order
+    if nbt == 0:                                                                 # and it is the library's choice
+        assert all(torch.equal(a, b_) for a, b_ in zip(npa.varlen_dwconv_bwd(xd, dyd, cud, wd), (dx3, dw3, db3)))
+
+
+def test_role_split_backward_serves_only_the_fused_request_and_only_where_it_is_built():
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 31, torch.bfloat16, torch.bfloat16, seed=3)
+    xd, cud, wd, dyd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV)
+    dx0, dw0, db0 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    dx1, dw1, db1 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=1))
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dw=False)           # partial requests: sliding-window
+    assert dw is None and db is None and torch.equal(dx, dx0)
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False)
+    assert dx is None and torch.equal(dw, dw1) and torch.equal(db, db1)
+    assert_red_close(dw0, dw1.double().cpu(), "dw")
+    with pytest.raises(RuntimeError):
+        npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False, tuning=_lib.Tuning(algo=3))
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 15, torch.bfloat16, torch.bfloat16, seed=4)
+    with pytest.raises(RuntimeError):                                             # K = 15 has no role-split kernel
+        npa.varlen_dwconv_bwd(x.to(DEV), dy.to(DEV), cu.to(DEV), w.to(DEV), tuning=_lib.Tuning(algo=3))
+    x, cu, w, b, dy = _random_case([40, 3], 64, 31, torch.bfloat16, torch.bfloat16, seed=5)   # rows too narrow
+    with pytest.raises(RuntimeError):
+        npa.varlen_dwconv_bwd(x.to(DEV), dy.to(DEV), cu.to(DEV), w.to(DEV), tuning=_lib.Tuning(algo=3))
+    _check_case(x, cu, w, b, dy, "narrow rows K=31")
