@@ -1,18 +1,25 @@
 // LDS-staged fused backward for K = 31 in which every wave computes and the two outputs have their own waves
 // (gfx950, wave64).
 //
-// At K = 31 the backward issues 62 FMAs per element and is bound by the vector ALU as much as by HBM. A SIMD issues
-// FMAs near its rate only when 4 of its waves are in an FMA stream at once (measured on a register-only loop: one
-// wave-instruction per 3.3 cycles with 2 waves per SIMD, per 2.4 with 4): that allows 128 registers per lane, where
-// one wave holding K weights and K dw sums per channel needs 166, and it rules out idle loader waves, which cost as
-// many registers as a compute wave. So here
-//   * every wave computes, and at the top of a tile issues its share of the direct global->LDS loads of the NEXT
-//     tile (dy with K-1 halo rows, x without) into the other buffer; the loads land while the tile is computed;
+// At K = 31 the backward issues 62 FMAs per element and is bound by the vector ALU. A SIMD issues FMAs near its rate
+// (one v_fmac_f32 per 2.1 - 2.4 cycles, measured on register-only loops) only while 4 of its waves are in an FMA
+// stream at once; one wave alone issues one per 5 cycles. That allows 128 registers per lane, where one wave holding K
+// weights and K dw sums per channel needs 166, and it rules out idle loader waves, which cost as many registers as a
+// compute wave. So here
 //   * the two outputs go to two kinds of wave that share the staged dy tile:
 //       role 0 (dx):    dx[t] = sum_m w[K-1-m] * dy[t-P+m]           holds K weights + RW row sums
 //       role 1 (dw/db): dw[K-1-m] += x[t] * dy[t-P+m], db += dy[t]   holds K tap sums + RW x rows
 //     Neither needs the other's registers, nothing is exchanged, and both run the same unrolled schedule over the
 //     RW+K-1 staged rows of their RW output rows. dx sums its taps in the order of the sliding-window kernel (same bits).
+//     Every SIMD runs two waves of each role (SplitShape::role_of).
+//   * every wave computes. The dx waves also issue the direct global->LDS loads of the NEXT tile (dy with K-1 halo
+//     rows, x without) into the other buffer, one load every few rows of their FMA schedule, and store an output row
+//     as soon as its last tap is in; the dw/db waves never wait on memory.
+//   * a wave lowers its priority as it advances through a tile, which keeps the 4 waves of a SIMD in step up to the
+//     tile's barrier (the one synchronisation per tile: next tile landed, this tile's buffer free).
+// Cycles per tile and SIMD at T = 131072, C = 2048, one sequence (s_memtime around the phases): 15300 with every wave
+// loading at the top of the tile, roles on separate SIMDs' worth of waves and no priorities; 13300 as built, of which
+// 11000 in the row schedules at 2.2 cycles per vector instruction (5100 per SIMD and tile, 3968 of them FMAs).
 // Tiles, rounds, slot rotation and XCD grouping are those of the other LDS-staged kernels (dwconv_lds_kernels.h);
 // dw/db leave the block as in those (row groups summed through LDS in fixed order, one slab per token block, then
 // dwconv_finalize_kernel). No atomics; every sum has a fixed order.
@@ -20,8 +27,8 @@
 // Sequence boundaries: a wave whose rows and taps all lie in one sequence runs unmasked. Otherwise it makes one pass
 // per sequence that owns some of its output rows, over the staged rows of that sequence: the dx role skips the other
 // rows by scalar branches and stores the sequence's output rows at the end of the pass; the dw role loads the x rows
-// of the sequence (zero for the others), skips chunks of staged rows that hold none of the sequence's and selects a
-// zero for single rows of another sequence inside a chunk.
+// of the sequence (zero for the others), skips chunks of staged rows that hold none of the sequence's and masks
+// single rows of another sequence inside a chunk (the mask rides on the bf16 -> fp32 conversion).
 //
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); tensor contract:
 // modeling.py:339,421-439 and collator.py:322-325,405-458.
@@ -36,6 +43,13 @@ struct SplitShape {
     static constexpr int P = (K - 1) / 2;
     static constexpr int NROLE = 2;
     static constexpr int NW = NCW * NROLE * NRG;           // waves per block (all compute)
+    // wave -> (role, index within the role). The waves of a block go to the 4 SIMDs of a CU round-robin, so the role
+    // changes within a residue class of the wave index mod 4: every SIMD then runs waves of both roles, and the
+    // role with less work leaves its issue slots to the other instead of idling two of the four SIMDs.
+    __device__ static constexpr int role_of(int wv) { return (wv >> 2) & 1; }
+    __device__ static constexpr int index_of(int wv) { return (wv & 3) | ((wv >> 3) << 2); }
+    __device__ static constexpr int wave_of(int role, int idx) { return (idx & 3) | (role << 2) | ((idx >> 2) << 3); }
+    static_assert(NW % 8 == 0, "roles alternate in groups of 4 waves");
     static constexpr int NT = NW * 64;
     static constexpr int R = RW * NRG;                     // output rows per tile
     static constexpr int NROWS = R + K - 1;                // staged dy rows per tile
@@ -47,35 +61,15 @@ struct SplitShape {
     static constexpr int X_BYTES = R * CB_BYTES;           // x tile, no halo
     static constexpr int BUF_BYTES = IN_BYTES + X_BYTES;
     static constexpr int LDS_BYTES = 2 * BUF_BYTES;
+    static constexpr int RPL = 64 / CPR;                   // staged rows per 1 KiB load (64 lanes x 16 bytes)
+    static constexpr int NLD_IN = (NROWS + RPL - 1) / RPL; // loads of a dy tile
+    static constexpr int NLD_X = (R + RPL - 1) / RPL;      // loads of an x tile
     static_assert(CB_BYTES == 256 || CB_BYTES == 512 || CB_BYTES == 1024, "a staged row is 16, 32 or 64 chunks");
     static_assert(NW <= 16, "at most 1024 threads per block");
     static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers must fit in LDS");
     static_assert(NJ * CB_BYTES <= 65536, "ds_read immediate offsets (a wave reads NJ rows from one base) are 16 bit");
     static_assert(NW * VEC * 64 * 4 <= LDS_BYTES, "the final reduction reuses the tile buffers");
 };
-
-// Stage rows first_row .. first_row+nrows-1 (clamped to [0,T)) x this block's column block of `src` into
-// `dst` (row pitch CB_BYTES): the tile is one run of nrows*CPR 16-byte chunks, chunk 64*i + lane belongs
-// to load i, and loads i = w0, w0 + nw, ... to this wave. A load covers 64/CPR adjacent rows, each lane
-// forming its own (clamped) row offset. Staged rows in [edge, nrows-edge) are read by no other tile.
-template <typename SH, int ONCE_AUX>
-__device__ __forceinline__ void stage_rows_flat(const void* __restrict__ src, char* dst, int first_row, int nrows, int T,
-                                                size_t row_bytes, int col_byte0, int valid_bytes, int w0, int nw, int lane,
-                                                int edge) {
-    constexpr int CPR = SH::CPR, RPL = 64 / CPR;          // rows per load
-    const int rb = first_row > 0 ? first_row : 0;
-    const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
-    const int rowb = (int)row_bytes;
-    const int lrow = lane / CPR, lchunk = lane % CPR;
-    const int nloads = (nrows + RPL - 1) / RPL;
-    for (int i = w0; i < nloads; i += nw) {
-        const int j = i * RPL + lrow;                    // staged row of this lane
-        const int voff = (clamp_row(first_row + j, T) - rb) * rowb + col_byte0 + lchunk * 16;
-        char* d = dst + i * 1024;                         // base of the load in LDS: lanes land 16 bytes apart
-        const bool once = i * RPL >= edge && i * RPL + RPL <= nrows - edge;
-        if (j < nrows && lchunk * 16 < valid_bytes) load_to_lds<ONCE_AUX>(rs, d, voff, 0, once);
-    }
-}
 
 // One lane's slice of a staged row, read with a volatile access: the compiler may neither hoist it out of its
 // place in the unrolled schedule (all reads of a tile at the top would need NJ registers) nor merge it with
@@ -109,8 +103,8 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
-    const int wc = wv % NCW;
-    const int rg = wv / (NCW * NROLE);
+    const int wc = SH::index_of(wv) % NCW;
+    const int rg = SH::index_of(wv) / NCW;
     int cb, tb;
     lds_block_coords(g, cb, tb);
     const int T = g.T, S = g.S, C = g.C;
@@ -127,27 +121,87 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     const int c0 = cb * SH::CB_CH + lc0;
     const int out_voff = c0 * E;
 
-    auto stage_tile = [&](char* buf, int t0) __attribute__((always_inline)) {
-        stage_rows_flat<SH, kLoadAuxOnceBwd>(in, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, wv, SH::NW, lane,
-                                             2 * P);
-        // the x loads start where the dy loads ended, so that both tensors spread over all waves
-        constexpr int NLD = (SH::NROWS + 64 / SH::CPR - 1) / (64 / SH::CPR);
-        const int w0x = (wv + SH::NW - NLD % SH::NW) % SH::NW;
-        stage_rows_flat<SH, kLoadAuxOnceBwdX>(other, buf + SH::IN_BYTES, t0, R, T, row_bytes, col_byte0, valid_bytes, w0x,
-                                              SH::NW, lane, 0);
+    // ---- staging: direct global->LDS loads of 1 KiB (64 lanes x 16 bytes = RPL adjacent rows of the column block) ----
+    // A tile is one run of 16-byte chunks, dy rows first (NLD_IN loads), then x rows (NLD_X loads); load number
+    // lw + n * NLW is the n-th of this wave. Each lane forms its own row offset. Rows outside [0, T) are not clamped:
+    // their offsets fall outside the descriptor (or, on a tensor beyond 4 GiB, on other rows of it), so nothing faults,
+    // and what lands in LDS for them is never used (a branch or a select, never a product, masks it).
+    // The dx role stages the tiles: its waves have less to do per tile than the dw/db role's (no x rows to read, no
+    // row masks), and a wave that stores dx and also waits for loads is the only kind that waits for store
+    // acknowledgements at the tile's barrier; the dw/db role never waits on memory.
+    constexpr bool LOADS = ROLE == 0;
+    constexpr int NLW = SH::NW / NROLE;                                         // waves that stage tiles
+    constexpr int NPW = (SH::NLD_IN + SH::NLD_X + NLW - 1) / NLW;               // loads per such wave and tile
+    // A loader wave issues its loads of the next tile one at a time, every SSTEP staged rows of its FMA schedule.
+    // (Issued all at once at the top of the tile they fill the CU's memory pipeline, and the wave stalls at their
+    // issue for a sixth of the tile: 2500 of 15000 cycles measured.)
+    constexpr int SSTEP = (NJ * 9 / 10) / NPW > 1 ? (NJ * 9 / 10) / NPW : 1;
+    static_assert(NPW * SSTEP <= NJ, "a slot for every load");
+    const int lw = rg * NCW + wc;                                               // this wave's index among them
+    const int lrow = lane / SH::CPR, lchunk = lane % SH::CPR;
+    const bool lane_ok = lchunk * 16 < valid_bytes;
+    rsrc_t rs_in, rs_x;         // descriptors of the tile being staged
+    int s_in = 0;               // byte offset of its first dy row from the descriptor's first row (negative in tile 0)
+    char* nbuf = lds_raw;
+    int lw_t = lw;              // lw, made opaque in every tile: see stage_begin
+    const int v_lane = lrow * rowb + col_byte0 + lchunk * 16;
+    auto stage_begin = [&](char* buf, int t0) __attribute__((always_inline)) {
+        const int rb = t0 - P > 0 ? t0 - P : 0;
+        rs_in = rows_rsrc(in, rb, T, row_bytes);
+        rs_x = rows_rsrc(other, t0, T, row_bytes);
+        s_in = (t0 - P - rb) * rowb;
+        nbuf = buf;
+        // everything a load derives from the wave's index is the same in every tile; computed once outside the tile
+        // loop it would occupy some 50 scalar registers (NPW loads x flags and offsets) and push others into spills
+        lw_t = lw;
+        asm volatile("" : "+s"(lw_t));
     };
+    auto stage_one = [&](int n) __attribute__((always_inline)) {
+        const int gi = lw_t + n * NLW;
+        if (gi < SH::NLD_IN) {
+            const bool once = gi * SH::RPL >= 2 * P && gi * SH::RPL + SH::RPL <= SH::NROWS - 2 * P;   // no other tile stages it
+            if (lane_ok && (SH::NROWS % SH::RPL == 0 || gi * SH::RPL + lrow < SH::NROWS))
+                load_to_lds<kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * rowb)), 0, once);
+        } else if (gi < SH::NLD_IN + SH::NLD_X) {
+            const int i = gi - SH::NLD_IN;
+            if (lane_ok && (R % SH::RPL == 0 || i * SH::RPL + lrow < R))
+                load_to_lds<kLoadAuxOnceBwdX>(rs_x, nbuf + SH::IN_BYTES + i * 1024, v_lane + i * (SH::RPL * rowb), 0, true);
+        }
+    };
+    bool spread = false;        // the loads of the next tile are issued from inside the row schedule
 
     // role 0: a[v][m] = w[K-1-m], the weight of staged row u + m for output row u;   b = row sums of dx
     // role 1: a[v][m] = sum over rows of x[t] * dy[t-P+m] (= dw[K-1-m]);              b = x rows
     float a[VEC][K];
     float b[RW][VEC];
-    float c[VEC];          // role 0: zero (what a row sum starts from); role 1: db
+    float c[VEC];          // role 1: db
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         c[v] = 0.f;
 #pragma unroll
         for (int m = 0; m < K; ++m) a[v][m] = 0.f;
     }
+    auto pin_a = [&](auto v_c, auto m_c) __attribute__((always_inline)) {
+        float& x = a[decltype(v_c)::value][decltype(m_c)::value];
+        asm volatile("" : "+v"(x) : : "memory");
+    };
+    auto pin_b = [&](auto u_c, auto v_c) __attribute__((always_inline)) {
+        float& x = b[decltype(u_c)::value][decltype(v_c)::value];
+        asm volatile("" : "+v"(x) : : "memory");
+    };
+    // the sums row j touches: role 0 b[u][*], role 1 a[*][j-u], for every output row u with a tap on row j
+    auto pin_row = [&](auto j_c) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_c)::value;
+        static_for<RW>([&](auto u_c) __attribute__((always_inline)) {
+            constexpr int u = decltype(u_c)::value;
+            if constexpr (j - u >= 0 && j - u < K) {
+                static_for<VEC>([&](auto v_c) __attribute__((always_inline)) {
+                    if constexpr (ROLE == 0) pin_b(u_c, v_c);
+                    else pin_a(v_c, std::integral_constant<int, j - u>{});
+                });
+            }
+        });
+    };
     if constexpr (ROLE == 0) {
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
@@ -160,19 +214,35 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             }
         }
     }
-    stage_tile(lds_raw, tb * R);
+    if constexpr (LOADS) {
+        stage_begin(lds_raw, tb * R);
+        for (int n = 0; n < NPW; ++n) stage_one(n);
+    }
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     int nce = 0;
     bool interior = wave_locate<RW, P>(sc, nce, cu, S, T, tb * R + rg * RW);
-    wait_vmem_all();       // this wave's share of the first tile has landed
+    if constexpr (LOADS) wait_vmem_all();       // this wave's share of the first tile has landed
     __syncthreads();
+
+    rsrc_t ro;                  // output rows of the wave in the current tile (dx role)
+    // slot of the schedule after staged row j: the next load of the tile being staged
+    auto slot = [&](auto j_c) __attribute__((always_inline)) {
+        constexpr int j = decltype(j_c)::value;
+        // A wave's priority falls as it advances through the tile (3 at the top, 0 in the last quarter), so the waves
+        // of a SIMD that lag behind catch up and all reach the tile's barrier together. The arbiter otherwise favours
+        // the same waves all the time, and the last one finishes alone at a quarter of the SIMD's issue rate.
+        constexpr int Q = (NJ + 3) / 4;
+        if constexpr (j % Q == Q - 1 && j / Q < 3) __builtin_amdgcn_s_setprio(2 - j / Q);
+        if constexpr (LOADS && j % SSTEP == 0 && j / SSTEP < NPW) {
+            if (spread) stage_one(j / SSTEP);
+        }
+    };
 
     // the unrolled schedule over staged rows [jlo, jhi) of the wave's window (all NJ rows when UNMASKED):
     // row j feeds output rows u = j-K+1 .. j with tap m = j - u
-    auto run_rows = [&](const char* lp, auto unmasked_c, auto role_c, int jlo, int jhi) __attribute__((always_inline)) {
+    auto run_rows = [&](const char* lp, auto unmasked_c, int jlo, int jhi) __attribute__((always_inline)) {
         constexpr bool UNMASKED = decltype(unmasked_c)::value;
-        constexpr int RROLE = decltype(role_c)::value;
         Row nxt[2];
         if constexpr (UNMASKED) {
             lds_read_pinned<BF16, VEC>(lp, nxt[0]);
@@ -192,43 +262,35 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                 } else {
                     lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, gr);
                 }
-                if (RROLE == 1 && j >= P && j < P + RW) {   // centre row of output row j - P
-#pragma unroll
-                    for (int v = 0; v < VEC; ++v) c[v] += gr[v];
-                }
 #pragma unroll
                 for (int u = 0; u < RW; ++u) {
                     if (j - u >= 0 && j - u < K) {
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) {
-                            if (RROLE == 0) b[u][v] = __builtin_fmaf(a[v][j - u], gr[v], b[u][v]);
-                            else a[v][j - u] = __builtin_fmaf(b[u][v], gr[v], a[v][j - u]);
-                        }
+                        for (int v = 0; v < VEC; ++v) b[u][v] = __builtin_fmaf(a[v][j - u], gr[v], b[u][v]);
                     }
                 }
                 // pin this row's arithmetic here: every sum it touched passes through an empty volatile asm, which
                 // is ordered with the (volatile) row reads, so the FMAs of row j stay between the reads of rows
                 // j + 2 and j + 3
                 if constexpr (UNMASKED) {
-#pragma unroll
-                    for (int u = 0; u < RW; ++u) {
-                        if (j - u >= 0 && j - u < K) {
-                            if (RROLE == 0) pin_regs<VEC>(b[u]);
-                            else {
-#pragma unroll
-                                for (int v = 0; v < VEC; ++v) asm volatile("" : "+v"(a[v][j - u]) : : "memory");
-                            }
-                        }
+                    pin_row(j_c);
+                    // output row j - (K-1) has all its taps: out it goes, long before the tile ends
+                    if constexpr (j >= K - 1) {
+                        Row o;
+                        o.from_f32(b[j - (K - 1)]);
+                        if (active) o.bstore(ro, out_voff, (j - (K - 1)) * rowb);
                     }
                 }
             }
+            if constexpr (UNMASKED) slot(j_c);
             __builtin_amdgcn_sched_barrier(0);
         });
     };
 
-    // dw role at a boundary: the staged rows in chunks of CH; a chunk with no row of the pass's sequence is skipped by one
-    // scalar branch, inside a chunk a row of another sequence contributes a selected zero. (One branch per row, as in
-    // the dx role, makes the register allocator keep two copies of the K tap sums per channel.)
+    // dw role: the staged rows in chunks of CH; a chunk with no row of the pass's sequence is skipped by one scalar
+    // branch, inside a chunk a row of another sequence contributes a selected zero. (One branch per row, as in the
+    // dx role, makes the register allocator keep two copies of the K tap sums per channel.) An interior tile is the
+    // single pass over all rows.
     auto run_rows_chunked = [&](const char* lp, int jlo, int jhi) __attribute__((always_inline)) {
         constexpr int CH = 12, NCH = (NJ + CH - 1) / CH;
         static_for<NCH>([&](auto ch_c) __attribute__((always_inline)) {
@@ -242,10 +304,19 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                     constexpr int j = j0 + decltype(jj_c)::value;
                     const bool in = j >= jlo && j < jhi;
                     float gr[VEC];
-                    nxt[(j - j0) & 1].to_f32(gr);
-                    if (j + 2 < j1) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[(j - j0) & 1]);
+                    if constexpr (BF16 && VEC == 2) {
+                        // the row mask rides on the bf16 -> fp32 conversion: the high half by an AND, the low half by a
+                        // byte permute, both with a wave-uniform (scalar) second operand chosen by `in`
+                        const uint32_t raw = nxt[(j - j0) & 1].d[0];
+                        gr[1] = __uint_as_float(raw & (in ? 0xffff0000u : 0u));
+                        gr[0] = __uint_as_float(__builtin_amdgcn_perm(raw, raw, in ? 0x01000c0cu : 0x0c0c0c0cu));
+                        if (j + 2 < j1) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[(j - j0) & 1]);
+                    } else {
+                        nxt[(j - j0) & 1].to_f32(gr);
+                        if (j + 2 < j1) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[(j - j0) & 1]);
 #pragma unroll
-                    for (int v = 0; v < VEC; ++v) gr[v] = in ? gr[v] : 0.f;
+                        for (int v = 0; v < VEC; ++v) gr[v] = in ? gr[v] : 0.f;
+                    }
                     if (j >= P && j < P + RW) {
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) c[v] += gr[v];
@@ -254,12 +325,11 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                     for (int u = 0; u < RW; ++u) {
                         if (j - u >= 0 && j - u < K) {
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) {
-                                a[v][j - u] = __builtin_fmaf(b[u][v], gr[v], a[v][j - u]);
-                                asm volatile("" : "+v"(a[v][j - u]) : : "memory");
-                            }
+                            for (int v = 0; v < VEC; ++v) a[v][j - u] = __builtin_fmaf(b[u][v], gr[v], a[v][j - u]);
                         }
                     }
+                    pin_row(std::integral_constant<int, j>{});
+                    slot(std::integral_constant<int, j>{});
                     __builtin_amdgcn_sched_barrier(0);
                 });
             }
@@ -272,13 +342,23 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         const int qn = lds_next_slot(g, q);
         char* cur = lds_raw + (it & 1) * SH::BUF_BYTES;
         const int rn = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
-        if (rn < T) stage_tile(lds_raw + ((it + 1) & 1) * SH::BUF_BYTES, rn);
         const int tf = t0 + rg * RW;
+        __builtin_amdgcn_s_setprio(3);
+        if constexpr (LOADS) {
+            // an interior wave runs every row of its schedule exactly once: its loads go into the schedule's slots
+            spread = rn < T && tf < T && interior;
+            if (rn < T) {
+                stage_begin(lds_raw + ((it + 1) & 1) * SH::BUF_BYTES, rn);
+                if (!spread) {
+                    for (int n = 0; n < NPW; ++n) stage_one(n);
+                }
+            }
+        }
         if (tf < T) {
             const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
             const char* lpi = cur + loff;                              // taps: staged row j <-> global row tf - P + j
             const char* lpx = cur + SH::IN_BYTES + loff;               // backward x: row u <-> global row tf + u
-            const rsrc_t ro = rows_rsrc(out, tf, T, row_bytes);
+            ro = rows_rsrc(out, tf, T, row_bytes);
             // role 0: store output rows [u0, u1) of the wave from b
             auto store_rows = [&](int u0, int u1) __attribute__((always_inline)) {
 #pragma unroll
@@ -293,9 +373,8 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
 #pragma unroll
                     for (int u = 0; u < RW; ++u)
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) b[u][v] = c[v];
-                    run_rows(lpi, std::true_type{}, std::integral_constant<int, 0>{}, 0, NJ);
-                    store_rows(0, RW);
+                        for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                    run_rows(lpi, std::true_type{}, 0, NJ);
                 } else {
                     SeqCursor sq = sc;                      // positioned on row tf
                     int u0 = 0;
@@ -309,8 +388,8 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
 #pragma unroll
                         for (int u = 0; u < RW; ++u)
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) b[u][v] = c[v];
-                        run_rows(lpi, std::false_type{}, std::integral_constant<int, 0>{}, jlo, jhi);
+                            for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                        run_rows(lpi, std::false_type{}, jlo, jhi);
                         store_rows(u0, u1);
                         u0 = u1;
                     }
@@ -332,11 +411,14 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                         u1 = __builtin_amdgcn_readfirstlane(u1 > RW ? RW : u1);
                     }
 #pragma unroll
-                    for (int u = 0; u < RW; ++u) {
-                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, b[u]);
-                        if (!(u >= u0 && u < u1)) {
+                    for (int u = 0; u < RW; ++u) lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, b[u]);
+                    if (!interior) {
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                        for (int u = 0; u < RW; ++u) {
+                            if (!(u >= u0 && u < u1)) {
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                            }
                         }
                     }
                     run_rows_chunked(lpi, jlo, jhi);
@@ -345,12 +427,12 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             }
         }
         if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
-        wait_vmem_all();   // this wave's share of the next tile has landed
+        if constexpr (LOADS) wait_vmem_all();   // this wave's share of the next tile has landed
         __syncthreads();   // so has everybody else's; this tile's buffer may be overwritten
         q = qn;
     }
 
-    // ---- block-level pass: sum the NRG row groups of each role-1 wave-column, group order 0,1,2,... ----
+    // ---- block-level pass: sum the NRG row groups of each wave-column, group order 0,1,2,... ----
     float* slab = partial + (size_t)tb * (K + 1) * C;
     float* red = reinterpret_cast<float*>(lds_raw);   // [NW][VEC][64]; the tiles are dead after the last barrier
 #pragma unroll
@@ -366,7 +448,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         if (ROLE == 1 && rg == 0) {
 #pragma unroll
             for (int j = 1; j < NRG; ++j) {
-                const int ow = (j * NROLE + 1) * NCW + wc;
+                const int ow = SH::wave_of(1, j * NCW + wc);
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
             }
@@ -385,7 +467,7 @@ template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
 __global__ void __launch_bounds__(NCW * 2 * NRG * 64)
 dwconv_bwd_split_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                         const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
-    if ((wave_id() / NCW) % 2 == 0) split_role<BF16, K, VEC, RW, NRG, NCW, 0>(dy, x, cu, w, dx, partial, g);
+    if (SplitShape<BF16, K, VEC, RW, NRG, NCW>::role_of(wave_id()) == 0) split_role<BF16, K, VEC, RW, NRG, NCW, 0>(dy, x, cu, w, dx, partial, g);
     else split_role<BF16, K, VEC, RW, NRG, NCW, 1>(dy, x, cu, w, dx, partial, g);
 }
 
