@@ -271,20 +271,20 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
     return hipErrorInvalidConfiguration;
 }
 
-// ---- role-split LDS-staged backward at K = 31 (dwconv_lds_split_kernels.h) ---------------------------
+// ---- role-split LDS-staged kernels at K = 31 (dwconv_lds_split_kernels.h) ----------------------------
 bool split_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     const int E = bf16 ? 2 : 4;
     if (!lds_split_kernel_size(K) || T < 1) return false;
     if (((long long)C * E) % 16 || align_bits % 16) return false;
-    const SplitShapeSel sh = lds_split_shape(bf16, K);
+    const SplitShapeSel sh = lds_split_shape(false, bf16, K);      // the column block is the same in both passes
     return (long long)C * E >= (long long)sh.ncw * 64 * sh.vec * E;
 }
-int make_split_plan(bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
+int make_split_plan(bool fwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
     LdsPlan p{};
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    const SplitShapeSel sh = lds_split_shape(bf16, K);
+    const SplitShapeSel sh = lds_split_shape(fwd, bf16, K);
     const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
     const long long row_bytes = (long long)C * E;
     p.R = sh.rw * sh.nrg;
@@ -294,7 +294,7 @@ int make_split_plan(bool bf16, long long T, int C, int K, const nplm_dwconv_tuni
     int nbt = tune->nbt > 0 ? tune->nbt : kNumCU / p.ncb;     // one block of 16 waves per CU
     if (nbt < 1) nbt = 1;
     if (nbt > p.ntiles) nbt = p.ntiles;
-    if (tune->nbt <= 0) {
+    if (tune->nbt <= 0 && !fwd) {
         const long long cap = (long long)(kSlabBudgetBytes / ((size_t)(K + 1) * C * sizeof(float)));
         if (nbt > cap && cap >= 1) nbt = (int)cap;
     }
@@ -317,10 +317,10 @@ int make_split_plan(bool bf16, long long T, int C, int K, const nplm_dwconv_tuni
 // the sliding-window one at C=2048) and a backward asked for dx alone or dw/db alone the sliding-window kernel,
 // like everything the LDS kernels are not built for (K = 15 backward, other sizes, narrow or unaligned rows).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
-    if (tune && tune->algo == 3) return (bwd && split_eligible(bf16, T, C, K, align_bits)) ? 3 : -NPLM_DWCONV_ETUNING;
+    if (tune && tune->algo == 3) return split_eligible(bf16, T, C, K, align_bits) ? 3 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 2) return lds_eligible(bf16, T, C, K, align_bits) ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
-    if (bwd && split_eligible(bf16, T, C, K, align_bits)) return 3;
+    if (split_eligible(bf16, T, C, K, align_bits)) return 3;
     return lds_preferred(bwd, bf16, T, C, K, align_bits) ? 2 : 1;
 }
 
@@ -387,6 +387,13 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
     hipStream_t s = (hipStream_t)stream;
     const int algo = choose_algo(false, tune, bf16, T, C, K, bits);
     if (algo < 0) return algo;
+    if (algo == 3) {
+        LdsPlan lp;
+        rc = make_split_plan(true, bf16, T, C, K, tune, &lp);
+        if (rc) return rc;
+        const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
+        return (int)launch_fwd_split_k31(bf16, la, make_lds_geo(lp, T, C, S, w_flags), dim3(lp.ncb * lp.nbt), s);
+    }
     if (algo == 2) {
         LdsPlan lp;
         rc = make_lds_plan(false, bf16, T, C, K, tune, &lp);
@@ -448,7 +455,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     }
     if (algo == 3) {
         LdsPlan lp;
-        rc = make_split_plan(bf16, T, C, K, tune, &lp);
+        rc = make_split_plan(false, bf16, T, C, K, tune, &lp);
         if (rc) return rc;
         const size_t slab_bytes = (size_t)(K + 1) * C * sizeof(float);
         if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab_bytes * (size_t)lp.nbt)
@@ -750,7 +757,7 @@ size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t 
     }
     if (split_eligible(bf16, T, C, K, 0)) {
         LdsPlan lp;
-        if (make_split_plan(bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
+        if (make_split_plan(false, bf16, T, C, K, nullptr, &lp) == 0 && lp.nbt > slabs) slabs = lp.nbt;
     }
     const size_t bytes = (size_t)slabs * (K + 1) * C * sizeof(float);
     return (bytes + 255) & ~(size_t)255;
@@ -763,7 +770,7 @@ int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype
     if (algo < 0) return 0;
     if (algo == 3) {
         LdsPlan lp;
-        if (make_split_plan(bf16, T, C, K, tune, &lp)) return 0;
+        if (make_split_plan(false, bf16, T, C, K, tune, &lp)) return 0;
         return lp.nbt;
     }
     if (algo == 2) {

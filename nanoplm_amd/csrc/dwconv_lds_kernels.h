@@ -343,6 +343,18 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     const int ntl = (g.ntiles + g.nbt - 1) / g.nbt;        // rounds of the grid, the same for every block
     const size_t in_row_bytes = GATED ? 2 * row_bytes : row_bytes;   // pitch of x (z when gated)
     auto stage_tile = [&](char* buf, int first_row) {
+        if constexpr (PREGATE) {
+            // Every staged row is loaded exactly once, by the loader wave that later rewrites it in place
+            // (gate_prepass takes rows lw, lw + NWL, ... as these loads do). stage_rows_fixed pads every wave to the
+            // same number of loads by loading the last row again: such a second copy, issued by another wave, can
+            // land after the row's owner has turned it into h, and put the raw u and g back.
+            static_assert(!PREGATE || SH::NPIECE == 1, "a staged row is one load");
+            stage_rows<SH, kLoadAuxOnceFwd>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC, NWL,
+                                            lane, 2 * P);
+            stage_rows<SH, kLoadAuxOnceFwd>(x, buf + SH::TILE_BYTES, first_row, SH::NROWS, T, in_row_bytes, rowb + col_byte0,
+                                            valid_bytes, wv - SH::NWC, NWL, lane, 2 * P);
+            return;
+        }
         stage_rows_fixed<SH, CNT, kLoadAuxOnceFwd>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
                                   NWL, lane, 2 * P);
         if constexpr (GATED)

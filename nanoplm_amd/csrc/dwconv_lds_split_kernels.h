@@ -37,38 +37,40 @@
 
 namespace nplm {
 
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
+// FWD: the forward (y from x), which is the dx role alone on every wave, with the taps in forward order and the bias.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD = false>
 struct SplitShape {
     static constexpr int E = BF16 ? 2 : 4;
     static constexpr int P = (K - 1) / 2;
-    static constexpr int NROLE = 2;
+    static constexpr int NROLE = FWD ? 1 : 2;
     static constexpr int NW = NCW * NROLE * NRG;           // waves per block (all compute)
     // wave -> (role, index within the role). The waves of a block go to the 4 SIMDs of a CU round-robin, so the role
     // changes within a residue class of the wave index mod 4: every SIMD then runs waves of both roles, and the
     // role with less work leaves its issue slots to the other instead of idling two of the four SIMDs.
-    __device__ static constexpr int role_of(int wv) { return (wv >> 2) & 1; }
-    __device__ static constexpr int index_of(int wv) { return (wv & 3) | ((wv >> 3) << 2); }
+    __device__ static constexpr int role_of(int wv) { return FWD ? 0 : (wv >> 2) & 1; }
+    __device__ static constexpr int index_of(int wv) { return FWD ? wv : (wv & 3) | ((wv >> 3) << 2); }
     __device__ static constexpr int wave_of(int role, int idx) { return (idx & 3) | (role << 2) | ((idx >> 2) << 3); }
-    static_assert(NW % 8 == 0, "roles alternate in groups of 4 waves");
+    static_assert(FWD || NW % 8 == 0, "roles alternate in groups of 4 waves");
     static constexpr int NT = NW * 64;
     static constexpr int R = RW * NRG;                     // output rows per tile
-    static constexpr int NROWS = R + K - 1;                // staged dy rows per tile
+    static constexpr int NROWS = R + K - 1;                // staged dy (forward: x) rows per tile
     static constexpr int NJ = RW + K - 1;                  // of which a wave reads this many
     static constexpr int CB_BYTES = NCW * 64 * VEC * E;    // bytes of a row in one column block
     static constexpr int CB_CH = NCW * 64 * VEC;
     static constexpr int CPR = CB_BYTES / 16;              // 16-byte chunks per staged row
     static constexpr int IN_BYTES = NROWS * CB_BYTES;      // dy tile
-    static constexpr int X_BYTES = R * CB_BYTES;           // x tile, no halo
+    static constexpr int X_BYTES = FWD ? 0 : R * CB_BYTES; // backward: x tile, no halo
     static constexpr int BUF_BYTES = IN_BYTES + X_BYTES;
     static constexpr int LDS_BYTES = 2 * BUF_BYTES;
     static constexpr int RPL = 64 / CPR;                   // staged rows per 1 KiB load (64 lanes x 16 bytes)
     static constexpr int NLD_IN = (NROWS + RPL - 1) / RPL; // loads of a dy tile
-    static constexpr int NLD_X = (R + RPL - 1) / RPL;      // loads of an x tile
+    static constexpr int NLD_X = FWD ? 0 : (R + RPL - 1) / RPL;   // loads of an x tile
     static_assert(CB_BYTES == 256 || CB_BYTES == 512 || CB_BYTES == 1024, "a staged row is 16, 32 or 64 chunks");
     static_assert(NW <= 16, "at most 1024 threads per block");
     static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers must fit in LDS");
     static_assert(NJ * CB_BYTES <= 65536, "ds_read immediate offsets (a wave reads NJ rows from one base) are 16 bit");
     static_assert(NW * VEC * 64 * 4 <= LDS_BYTES, "the final reduction reuses the tile buffers");
+    static_assert(NW == 16, "4 waves per SIMD and one block per CU");
 };
 
 // One lane's slice of a staged row, read with a volatile access: the compiler may neither hoist it out of its
@@ -91,12 +93,13 @@ __device__ __forceinline__ void lds_read_pinned(const char* p, RowVec<BF16, VEC>
 // are two instantiations that share no variable, so that the register allocator treats them apart (one function
 // with both roles' K per-channel values meeting at every join needs 170 registers where either role needs 106).
 // Both execute the same sequence of barriers.
-// in = dy, other = x, out = dx, partial = dw/db slabs.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int ROLE>
+// Backward: in = dy, other = x, out = dx, partial = dw/db slabs. Forward: in = x, out = y, bias may be null.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD, int ROLE>
 __device__ __forceinline__ void split_role(const void* __restrict__ in, const void* __restrict__ other,
                                            const int32_t* __restrict__ cu, const void* __restrict__ w,
-                                           void* __restrict__ out, float* __restrict__ partial, const LdsGeo& g) {
-    using SH = SplitShape<BF16, K, VEC, RW, NRG, NCW>;
+                                           const void* __restrict__ bias, void* __restrict__ out,
+                                           float* __restrict__ partial, const LdsGeo& g) {
+    using SH = SplitShape<BF16, K, VEC, RW, NRG, NCW, FWD>;
     constexpr int P = SH::P, E = SH::E, R = SH::R, NJ = SH::NJ, NROLE = SH::NROLE;
     using Row = RowVec<BF16, VEC>;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
@@ -129,6 +132,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     // The dx role stages the tiles: its waves have less to do per tile than the dw/db role's (no x rows to read, no
     // row masks), and a wave that stores dx and also waits for loads is the only kind that waits for store
     // acknowledgements at the tile's barrier; the dw/db role never waits on memory.
+    // (In the forward every wave is of that kind.)
     constexpr bool LOADS = ROLE == 0;
     constexpr int NLW = SH::NW / NROLE;                                         // waves that stage tiles
     constexpr int NPW = (SH::NLD_IN + SH::NLD_X + NLW - 1) / NLW;               // loads per such wave and tile
@@ -148,7 +152,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     auto stage_begin = [&](char* buf, int t0) __attribute__((always_inline)) {
         const int rb = t0 - P > 0 ? t0 - P : 0;
         rs_in = rows_rsrc(in, rb, T, row_bytes);
-        rs_x = rows_rsrc(other, t0, T, row_bytes);
+        if constexpr (!FWD) rs_x = rows_rsrc(other, t0, T, row_bytes);
         s_in = (t0 - P - rb) * rowb;
         nbuf = buf;
         // everything a load derives from the wave's index is the same in every tile; computed once outside the tile
@@ -161,7 +165,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         if (gi < SH::NLD_IN) {
             const bool once = gi * SH::RPL >= 2 * P && gi * SH::RPL + SH::RPL <= SH::NROWS - 2 * P;   // no other tile stages it
             if (lane_ok && (SH::NROWS % SH::RPL == 0 || gi * SH::RPL + lrow < SH::NROWS))
-                load_to_lds<kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * rowb)), 0, once);
+                load_to_lds<FWD ? kLoadAuxOnceFwd : kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * rowb)), 0, once);
         } else if (gi < SH::NLD_IN + SH::NLD_X) {
             const int i = gi - SH::NLD_IN;
             if (lane_ok && (R % SH::RPL == 0 || i * SH::RPL + lrow < R))
@@ -174,7 +178,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     // role 1: a[v][m] = sum over rows of x[t] * dy[t-P+m] (= dw[K-1-m]);              b = x rows
     float a[VEC][K];
     float b[RW][VEC];
-    float c[VEC];          // role 1: db
+    float c[VEC];          // role 1: db; forward: the bias (what a row sum starts from); role 0 of the backward: zero
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         c[v] = 0.f;
@@ -207,11 +211,12 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         for (int v = 0; v < VEC; ++v) {
 #pragma unroll
             for (int m = 0; m < K; ++m) {
-                const size_t wi = (size_t)(c0 + v) * K + (K - 1 - m);
+                const size_t wi = (size_t)(c0 + v) * K + (FWD ? m : K - 1 - m);
                 float t = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[wi]) : reinterpret_cast<const float*>(w)[wi];
                 if (m == P && (g.w_flags & W_RESIDUAL)) t += 1.f;
                 a[v][m] = t;
             }
+            if (FWD && bias) c[v] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(bias)[c0 + v]) : reinterpret_cast<const float*>(bias)[c0 + v];
         }
     }
     if constexpr (LOADS) {
@@ -373,7 +378,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
 #pragma unroll
                     for (int u = 0; u < RW; ++u)
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                        for (int v = 0; v < VEC; ++v) b[u][v] = c[v];
                     run_rows(lpi, std::true_type{}, 0, NJ);
                 } else {
                     SeqCursor sq = sc;                      // positioned on row tf
@@ -388,7 +393,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
 #pragma unroll
                         for (int u = 0; u < RW; ++u)
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) b[u][v] = 0.f;
+                            for (int v = 0; v < VEC; ++v) b[u][v] = c[v];
                         run_rows(lpi, std::false_type{}, jlo, jhi);
                         store_rows(u0, u1);
                         u0 = u1;
@@ -432,6 +437,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         q = qn;
     }
 
+    if constexpr (FWD) return;
     // ---- block-level pass: sum the NRG row groups of each wave-column, group order 0,1,2,... ----
     float* slab = partial + (size_t)tb * (K + 1) * C;
     float* red = reinterpret_cast<float*>(lds_raw);   // [NW][VEC][64]; the tiles are dead after the last barrier
@@ -467,8 +473,17 @@ template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
 __global__ void __launch_bounds__(NCW * 2 * NRG * 64)
 dwconv_bwd_split_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                         const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
-    if (SplitShape<BF16, K, VEC, RW, NRG, NCW>::role_of(wave_id()) == 0) split_role<BF16, K, VEC, RW, NRG, NCW, 0>(dy, x, cu, w, dx, partial, g);
-    else split_role<BF16, K, VEC, RW, NRG, NCW, 1>(dy, x, cu, w, dx, partial, g);
+    if (SplitShape<BF16, K, VEC, RW, NRG, NCW>::role_of(wave_id()) == 0)
+        split_role<BF16, K, VEC, RW, NRG, NCW, false, 0>(dy, x, cu, w, nullptr, dx, partial, g);
+    else
+        split_role<BF16, K, VEC, RW, NRG, NCW, false, 1>(dy, x, cu, w, nullptr, dx, partial, g);
+}
+
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
+__global__ void __launch_bounds__(NCW * NRG * 64)
+dwconv_fwd_split_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
+                        const void* __restrict__ bias, void* __restrict__ y, const LdsGeo g) {
+    split_role<BF16, K, VEC, RW, NRG, NCW, true, 0>(x, nullptr, cu, w, bias, y, nullptr, g);
 }
 
 }  // namespace nplm

@@ -369,12 +369,14 @@ def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
     assert torch.equal(outs[0][0], outs[1][0])
     if outs[1][1] is not None:
         assert torch.equal(outs[0][1], outs[1][1])
-    if K == 31:                      # the role-split LDS-staged backward rotates its tile slots the same way
-        dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    if K == 31:                      # the role-split LDS-staged kernels rotate their tile slots the same way
+        tf = _lib.Tuning(algo=3, nbt=nbt)
+        assert torch.equal(npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=tf), outs[0][0])
+        dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=tf)
         assert torch.equal(dx, outs[0][1])
 
 
-# ---- role-split LDS-staged backward (K = 31) ---------------------------------------------------------
+# ---- role-split LDS-staged kernels (K = 31) -----------------------------------------------------------
 LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 16, 17, 30, 31, 32, 33, 700, 1, 1, 1,
               29, 0, 0, 45, 1200, 14]
 
@@ -383,15 +385,24 @@ LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 1
                                   (1152, torch.bfloat16), (2048, torch.bfloat16), (2056, torch.bfloat16),
                                   (128, torch.float32), (388, torch.float32), (1024, torch.float32)])
 @pytest.mark.parametrize("nbt", [0, 1, 5])
-def test_role_split_backward_matches_the_sliding_window_kernel_and_the_oracle(C, dt, nbt):
+def test_role_split_kernels_match_the_sliding_window_kernels_and_the_oracle(C, dt, nbt):
     """A fused K = 31 backward is served by a kernel whose waves are split into a dx role and a dw/db role over the
-    same LDS tiles. Sequences shorter than the 15-row halo, tile-edge lengths, empty sequences, partial column
-    blocks and one or a few blocks walking every tile: dx must equal the sliding-window kernel's bit for bit, and
-    dw/db the oracle's to the reduction tolerance."""
+    same LDS tiles, the K = 31 forward by the dx role alone. Sequences shorter than the 15-row halo, tile-edge
+    lengths, empty sequences, partial column blocks and one or a few blocks walking every tile: y and dx must equal
+    the sliding-window kernels' bit for bit, and dw/db the oracle's to the reduction tolerance."""
     print(f"[case] C={C} {dt} nbt={nbt}", flush=True)
     x, cu, w, b, dy = _random_case(LENS_SPLIT, C, 31, dt, dt, seed=C + nbt)
+    y64 = O.c_oracle_fwd(x, cu, w, b)
     dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
-    xd, cud, wd, dyd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV)
+    xd, cud, wd, dyd, bd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV), b.to(DEV)
+    for bias, res in ((bd, False), (None, False), (bd, True)):
+        y1 = npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res, tuning=_lib.Tuning(algo=1))
+        y3 = npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res, tuning=_lib.Tuning(algo=3, nbt=nbt))
+        assert torch.equal(y3, y1)
+        if nbt == 0:
+            assert torch.equal(npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res), y3)
+        if bias is not None and not res:
+            assert_act_close(y3, y64, dt, "y")
     dx1, dw1, db1 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=1))
     dx3, dw3, db3 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
     assert torch.equal(dx3, dx1)
@@ -405,7 +416,7 @@ def test_role_split_backward_matches_the_sliding_window_kernel_and_the_oracle(C,
         assert all(torch.equal(a, b_) for a, b_ in zip(npa.varlen_dwconv_bwd(xd, dyd, cud, wd), (dx3, dw3, db3)))
 
 
-def test_role_split_backward_serves_only_the_fused_request_and_only_where_it_is_built():
+def test_role_split_kernels_serve_only_what_they_are_built_for():
     x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 31, torch.bfloat16, torch.bfloat16, seed=3)
     xd, cud, wd, dyd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV)
     dx0, dw0, db0 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
@@ -420,7 +431,11 @@ def test_role_split_backward_serves_only_the_fused_request_and_only_where_it_is_
     x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 15, torch.bfloat16, torch.bfloat16, seed=4)
     with pytest.raises(RuntimeError):                                             # K = 15 has no role-split kernel
         npa.varlen_dwconv_bwd(x.to(DEV), dy.to(DEV), cu.to(DEV), w.to(DEV), tuning=_lib.Tuning(algo=3))
+    with pytest.raises(RuntimeError):
+        npa.varlen_dwconv_fwd(x.to(DEV), cu.to(DEV), w.to(DEV), None, tuning=_lib.Tuning(algo=3))
     x, cu, w, b, dy = _random_case([40, 3], 64, 31, torch.bfloat16, torch.bfloat16, seed=5)   # rows too narrow
     with pytest.raises(RuntimeError):
         npa.varlen_dwconv_bwd(x.to(DEV), dy.to(DEV), cu.to(DEV), w.to(DEV), tuning=_lib.Tuning(algo=3))
+    with pytest.raises(RuntimeError):
+        npa.varlen_dwconv_fwd(x.to(DEV), cu.to(DEV), w.to(DEV), None, tuning=_lib.Tuning(algo=3))
     _check_case(x, cu, w, b, dy, "narrow rows K=31")
