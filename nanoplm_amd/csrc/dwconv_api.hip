@@ -310,17 +310,20 @@ int make_split_plan(bool fwd, bool bf16, long long T, int C, int K, const nplm_d
 }
 
 // algo requested by the caller (0 = library's choice) -> 1 sliding-window, 2 LDS-staged, 3 role-split LDS-staged.
-// Measured on MI355X at T=131072, C=1024, K=7, bf16: both passes are fastest LDS-staged (the chip
-// sweeps one compact window of rows with every load of a tile issued at once). At K=31 (ALU-bound)
-// the LDS-staged forward still wins by ~17 % (C=1024 and 2048); one wave cannot hold the fused backward's
-// registers there, so the backward that produces every output takes the role-split kernel (13 - 15 % faster than
-// the sliding-window one at C=2048) and a backward asked for dx alone or dw/db alone the sliding-window kernel,
-// like everything the LDS kernels are not built for (K = 15 backward, other sizes, narrow or unaligned rows).
+// Measured on MI355X, bf16, T=131072:
+//   K=7, C=1024: both passes are fastest LDS-staged (the chip sweeps one compact window of rows with every load of a
+//     tile issued at once).
+//   K=31 and K=15 backward (ALU-bound; one wave cannot hold the fused backward's registers): the role-split kernel,
+//     when every output is asked for - C=2048, K=31: 510 us against 720 sliding-window on the log-normal length mix;
+//     K=15: 345 against 385 (C=1024: 177 against 205). A backward asked for dx alone or dw/db alone takes the
+//     sliding-window kernel, like everything the LDS kernels are not built for (other sizes, narrow or unaligned rows).
+//   K=31 forward: the role-split kernel's dx role on every wave, 262 us against 299 LDS-staged with loader waves (C=2048).
+//   K=15 forward: LDS-staged with loader waves, 190 us against 203 role-split and 227 sliding-window (C=2048).
 int choose_algo(bool bwd, const nplm_dwconv_tuning* tune, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     if (tune && tune->algo == 3) return split_eligible(bf16, T, C, K, align_bits) ? 3 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 2) return lds_eligible(bf16, T, C, K, align_bits) ? 2 : -NPLM_DWCONV_ETUNING;
     if (tune && tune->algo == 1) return 1;
-    if (split_eligible(bf16, T, C, K, align_bits)) return 3;
+    if (split_eligible(bf16, T, C, K, align_bits) && (bwd || K == 31)) return 3;
     return lds_preferred(bwd, bf16, T, C, K, align_bits) ? 2 : 1;
 }
 
@@ -392,7 +395,9 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
         rc = make_split_plan(true, bf16, T, C, K, tune, &lp);
         if (rc) return rc;
         const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
-        return (int)launch_fwd_split_k31(bf16, la, make_lds_geo(lp, T, C, S, w_flags), dim3(lp.ncb * lp.nbt), s);
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, w_flags);
+        return (int)(K == 31 ? launch_fwd_split_k31(bf16, la, lg, dim3(lp.ncb * lp.nbt), s)
+                             : launch_fwd_split_k15(bf16, la, lg, dim3(lp.ncb * lp.nbt), s));
     }
     if (algo == 2) {
         LdsPlan lp;
@@ -464,7 +469,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         const ConvPtrs la{x, dy, cu, w, nullptr, dx, part};
         const LdsGeo lg = make_lds_geo(lp, T, C, S, w_flags);
         const dim3 grid(lp.ncb * lp.nbt);
-        hipError_t e = launch_bwd_split_k31(bf16, la, lg, grid, s);
+        hipError_t e = K == 31 ? launch_bwd_split_k31(bf16, la, lg, grid, s) : launch_bwd_split_k15(bf16, la, lg, grid, s);
         if (e != hipSuccess) return (int)e;
         if (tune && tune->mid_event) {
             e = hipEventRecord((hipEvent_t)tune->mid_event, s);

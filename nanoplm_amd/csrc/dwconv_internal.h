@@ -116,6 +116,8 @@ hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, c
 // role-split LDS kernels at K = 31 (fixed shape per dtype, see lds_split_shape())
 hipError_t launch_bwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_bwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_fwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
 NPLM_DECLARE_LDS_K(7)
@@ -167,18 +169,19 @@ constexpr LdsShapeSel lds_default_shape(bool bwd, bool bf16, int K) {
         return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 8, 2, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
     return bwd ? LdsShapeSel{bf16, bf16 ? 2 : 1, 10, 3, 4, 4, 2} : LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 4, 2, 4, 2};
 }
-// Role-split LDS kernels at K = 31 (dwconv_lds_split_kernels.h): 512-byte column blocks (2 wave-columns x 4 bytes per
-// lane), 16 waves of 16 rows that all compute.
-//   backward: 4 row groups x 2 roles, 64-row tiles, two (dy tile of 64 + K-1 rows, x tile of 64 rows) pairs = 158 KiB.
-//     T=131072, bf16, backward + finalize in us, sliding-window kernel -> this one: C=2048 one long sequence 677 -> 465,
-//     lengths 20 - 512 663 -> 500, the log-normal mix 720 -> 510; C=1024 lengths 20 - 512 376 -> 278.
-//   forward: 8 row groups, 128-row tiles, two x tiles of 128 + K-1 rows = 158 KiB.
-// At K = 15 the first version of the backward (every wave loading at the top of a tile) was no faster than the
-// sliding-window kernel (195 against 195 us at C=1024); K = 15 is not built.
+// Role-split LDS kernels at K = 31 and 15 (dwconv_lds_split_kernels.h): 512-byte column blocks (2 wave-columns x 4
+// bytes per lane), 16 waves of 16 rows that all compute.
+//   backward: 4 row groups x 2 roles, 64-row tiles, two (dy tile of 64 + K-1 rows, x tile of 64 rows) pairs (158 KiB
+//     at K = 31).
+//     T=131072, bf16, backward + finalize in us, sliding-window kernel -> this one: K=31, C=2048: one long sequence
+//     677 -> 465, lengths 20 - 512 663 -> 500, the log-normal mix 720 -> 510; C=1024 lengths 20 - 512 376 -> 278.
+//     K=15, C=2048: 354 -> 306, 390 -> 339, 385 -> 345; C=1024: 186 -> 156, 205 -> 180, 205 -> 177.
+//   forward: 8 row groups, 128-row tiles, two x tiles of 128 + K-1 rows (158 KiB at K = 31). The library's choice
+//     at K = 31 only: at K = 15 the forward with loader waves is faster (C=2048: 190 against 203 us).
 struct SplitShapeSel {
     int vec, rw, nrg, ncw;
 };
-constexpr bool lds_split_kernel_size(int K) { return K == 31; }
+constexpr bool lds_split_kernel_size(int K) { return K == 31 || K == 15; }
 constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
     (void)K;
     return SplitShapeSel{bf16 ? 2 : 1, 16, fwd ? 8 : 4, 2};

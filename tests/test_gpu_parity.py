@@ -369,14 +369,14 @@ def test_equal_length_sequences_on_rotating_tile_slots(K, C, dt, seq_len, nbt):
     assert torch.equal(outs[0][0], outs[1][0])
     if outs[1][1] is not None:
         assert torch.equal(outs[0][1], outs[1][1])
-    if K == 31:                      # the role-split LDS-staged kernels rotate their tile slots the same way
+    if K in (15, 31):                # the role-split LDS-staged kernels rotate their tile slots the same way
         tf = _lib.Tuning(algo=3, nbt=nbt)
         assert torch.equal(npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=tf), outs[0][0])
         dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=tf)
         assert torch.equal(dx, outs[0][1])
 
 
-# ---- role-split LDS-staged kernels (K = 31) -----------------------------------------------------------
+# ---- role-split LDS-staged kernels (K = 31, 15) -------------------------------------------------------
 LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 16, 17, 30, 31, 32, 33, 700, 1, 1, 1,
               29, 0, 0, 45, 1200, 14]
 
@@ -385,13 +385,14 @@ LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 1
                                   (1152, torch.bfloat16), (2048, torch.bfloat16), (2056, torch.bfloat16),
                                   (128, torch.float32), (388, torch.float32), (1024, torch.float32)])
 @pytest.mark.parametrize("nbt", [0, 1, 5])
-def test_role_split_kernels_match_the_sliding_window_kernels_and_the_oracle(C, dt, nbt):
-    """A fused K = 31 backward is served by a kernel whose waves are split into a dx role and a dw/db role over the
-    same LDS tiles, the K = 31 forward by the dx role alone. Sequences shorter than the 15-row halo, tile-edge
-    lengths, empty sequences, partial column blocks and one or a few blocks walking every tile: y and dx must equal
-    the sliding-window kernels' bit for bit, and dw/db the oracle's to the reduction tolerance."""
-    print(f"[case] C={C} {dt} nbt={nbt}", flush=True)
-    x, cu, w, b, dy = _random_case(LENS_SPLIT, C, 31, dt, dt, seed=C + nbt)
+@pytest.mark.parametrize("K", [31, 15])
+def test_role_split_kernels_match_the_sliding_window_kernels_and_the_oracle(K, C, dt, nbt):
+    """A fused K = 31 or 15 backward is served by a kernel whose waves are split into a dx role and a dw/db role over
+    the same LDS tiles, the K = 31 forward by the dx role alone (at K = 15 on request). Sequences shorter than the
+    halo, tile-edge lengths, empty sequences, partial column blocks and one or a few blocks walking every tile: y
+    and dx must equal the sliding-window kernels' bit for bit, and dw/db the oracle's to the reduction tolerance."""
+    print(f"[case] K={K} C={C} {dt} nbt={nbt}", flush=True)
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, C, K, dt, dt, seed=C + nbt + K)
     y64 = O.c_oracle_fwd(x, cu, w, b)
     dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
     xd, cud, wd, dyd, bd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV), b.to(DEV)
@@ -399,7 +400,7 @@ def test_role_split_kernels_match_the_sliding_window_kernels_and_the_oracle(C, d
         y1 = npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res, tuning=_lib.Tuning(algo=1))
         y3 = npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res, tuning=_lib.Tuning(algo=3, nbt=nbt))
         assert torch.equal(y3, y1)
-        if nbt == 0:
+        if nbt == 0:                                                             # (K = 15: the LDS-staged forward)
             assert torch.equal(npa.varlen_dwconv_fwd(xd, cud, wd, bias, residual=res), y3)
         if bias is not None and not res:
             assert_act_close(y3, y64, dt, "y")
@@ -428,8 +429,8 @@ def test_role_split_kernels_serve_only_what_they_are_built_for():
     assert_red_close(dw0, dw1.double().cpu(), "dw")
     with pytest.raises(RuntimeError):
         npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False, tuning=_lib.Tuning(algo=3))
-    x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 15, torch.bfloat16, torch.bfloat16, seed=4)
-    with pytest.raises(RuntimeError):                                             # K = 15 has no role-split kernel
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, 512, 9, torch.bfloat16, torch.bfloat16, seed=4)
+    with pytest.raises(RuntimeError):                                             # K = 9 has no role-split kernel
         npa.varlen_dwconv_bwd(x.to(DEV), dy.to(DEV), cu.to(DEV), w.to(DEV), tuning=_lib.Tuning(algo=3))
     with pytest.raises(RuntimeError):
         npa.varlen_dwconv_fwd(x.to(DEV), cu.to(DEV), w.to(DEV), None, tuning=_lib.Tuning(algo=3))
