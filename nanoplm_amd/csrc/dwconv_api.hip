@@ -183,7 +183,7 @@ bool lds_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
 // to 11/20; the sliding-window kernels win otherwise.
 bool lds_preferred(bool bwd, bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     if (!lds_eligible(bf16, T, C, K, align_bits)) return false;
-    if (K > 9 && bwd) return false;        // K = 15, 31: only the forward is built (the fused backward does not fit its registers)
+    if (K > 9 && bwd) return false;        // K = 15, 31: no single-role LDS backward (it does not fit the registers); see split_eligible
     const long long E = bf16 ? 2 : 4;
     const long long row_bytes = (long long)C * E;
     const LdsShapeSel sh = lds_shape_for(bwd, bf16, K, row_bytes);
@@ -271,7 +271,7 @@ hipError_t launch_bwd_lds(int K, const LdsPlan& p, bool wdx, bool wdw, const Con
     return hipErrorInvalidConfiguration;
 }
 
-// ---- role-split LDS-staged kernels at K = 31 (dwconv_lds_split_kernels.h) ----------------------------
+// ---- role-split LDS-staged kernels at K = 31 and 15 (dwconv_lds_split_kernels.h) ---------------------
 bool split_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     const int E = bf16 ? 2 : 4;
     if (!lds_split_kernel_size(K) || T < 1) return false;
