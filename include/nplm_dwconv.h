@@ -173,6 +173,23 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
                           int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
+ * LayerNorm fused into the forward, for a conv that takes the place of a sub-module of the reference's pre-norm
+ * encoder layer (ModernBertEncoderLayer.forward, modeling.py:404-414: `x + attn(attn_norm(x))`, the norm being a
+ * torch.nn.LayerNorm over the hidden dimension, modeling.py:264-266):
+ *   n = layer_norm(x; ln_weight, ln_bias, eps) over the C channels of a row (statistics and n in fp32, never stored)
+ *   y = conv(n; w, b)            (+ x with NPLM_DWCONV_RESIDUAL: the identity is the raw x, not n)
+ *   stats (optional, may be NULL): [T][2] fp32, (mean, rstd) of every row - what a LayerNorm backward needs
+ * x, y: act_dtype; ln_weight, ln_bias (may be NULL), w, b (may be NULL): w_dtype.
+ * Built for K in {3,5,7,9} and rows that fit one 2 KiB column block (C * elemsize <= 2048 and a multiple of 16 bytes,
+ * 16-byte aligned x / y), so that a block sees whole rows; anything else returns -NPLM_DWCONV_EUNSUPPORTED and
+ * launches nothing (callers then run LayerNorm and nplm_dwconv_fwd_ex).
+ */
+int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, const void* ln_bias, float eps,
+                       const void* w, const void* b, void* y, float* stats,
+                       int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
+
+/*
  * Debug helper: copies cu to the host (synchronises `stream`) and verifies the preconditions.
  * Returns 0, -NPLM_DWCONV_ECU, another argument error, or a hipError_t.
  */

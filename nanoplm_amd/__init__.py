@@ -27,6 +27,12 @@ from .gated import (  # noqa: F401
     gated_supported,
     gated_varlen_dwconv,
 )
+from .lnconv import (  # noqa: F401
+    LnVarlenDWConv1dFunction,
+    ln_dwconv_fwd,
+    ln_supported,
+    ln_varlen_dwconv,
+)
 from .hygiene import conv_parameters, split_conv_parameters  # noqa: F401
 
 __version__ = "0.1.0"

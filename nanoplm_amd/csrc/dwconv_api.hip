@@ -635,6 +635,47 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     return -NPLM_DWCONV_EUNSUPPORTED;
 }
 
+// ---- LayerNorm-fused forward (dwconv_ln_kernels.h) ---------------------------------------------------
+int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, const void* ln_bias, float eps,
+                       const void* w, const void* b, void* y, float* stats, int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    if (T == 0) return 0;
+    if (!x || !cu || !w || !y || !ln_weight) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t E = bf16 ? 2 : 4;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if (((uintptr_t)w | (uintptr_t)b | (uintptr_t)ln_weight | (uintptr_t)ln_bias) % WE || (uintptr_t)cu % 4 ||
+        (uintptr_t)stats % 4 || ((uintptr_t)x | (uintptr_t)y) % E)
+        return -NPLM_DWCONV_EALIGN;
+    const long long row_bytes = (long long)C * (long long)E;
+    if (!lds_ln_kernel_size(K) || row_bytes % 16 || row_bytes > kLnCbBytes || ((uintptr_t)x | (uintptr_t)y) % 16)
+        return -NPLM_DWCONV_EUNSUPPORTED;
+    LdsPlan lp{};
+    lp.sh = lds_ln_shape(bf16);
+    lp.R = lp.sh.rw * lp.sh.nrg;
+    lp.ncb = 1;
+    lp.ntiles = ceil_div(T, lp.R);
+    lp.nbt = lp.ntiles < kNumCU ? lp.ntiles : kNumCU;          // one block of 16 waves and three tiles per CU
+    lp.xcd_group = (lp.nbt % (kNumXCD * 8) == 0) ? 8 : 0;
+    lp.rot_step = lp.nbt > 2 ? (int)((long long)lp.nbt * 618 / 1000) | 1 : 0;
+    if (lp.rot_step >= lp.nbt) lp.rot_step = lp.nbt - 1;
+    const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
+    const LnArgs ln{ln_weight, ln_bias, stats, eps};
+    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+    const dim3 grid(lp.nbt);
+    hipStream_t s = (hipStream_t)stream;
+    switch (K) {
+        case 3: return (int)launch_ln_fwd_k3(bf16, la, ln, g, grid, s);
+        case 5: return (int)launch_ln_fwd_k5(bf16, la, ln, g, grid, s);
+        case 7: return (int)launch_ln_fwd_k7(bf16, la, ln, g, grid, s);
+        case 9: return (int)launch_ln_fwd_k9(bf16, la, ln, g, grid, s);
+    }
+    return -NPLM_DWCONV_EUNSUPPORTED;
+}
+
 size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;

@@ -8,6 +8,7 @@
 #include "dwconv_kernels.h"
 #include "dwconv_lds_kernels.h"
 #include "dwconv_lds_split_kernels.h"
+#include "dwconv_ln_kernels.h"
 
 #ifdef __cplusplus
 extern "C" {
@@ -117,6 +118,11 @@ hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, c
 hipError_t launch_bwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_bwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+// LayerNorm-fused forward (dwconv_ln_kernels.h), K <= 9, fixed shape per dtype, see lds_ln_shape()
+hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)
@@ -186,6 +192,14 @@ constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
     (void)K;
     return SplitShapeSel{bf16 ? 2 : 1, 16, fwd ? 8 : 4, 2};
 }
+// LayerNorm-fused forward: one 2 KiB column block holds a whole row (C <= 1024 in bf16, 512 in fp32); 4 wave-columns x 8
+// bytes per lane, 2 row groups of 8 rows (16-row tiles of K + 15 staged rows), 8 compute + 8 loader waves, three tiles
+// (one computed, one having its row statistics taken by the loader waves, one in flight: 132 KiB at K = 7). With two
+// 24-row tiles nothing is in flight while the statistics of a tile are taken, and the forward runs at 148 us instead of
+// 115 - 120 us (T=131072, C=1024, K=7, bf16).
+constexpr bool lds_ln_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+constexpr int kLnCbBytes = 2048;
+constexpr LdsShapeSel lds_ln_shape(bool bf16) { return LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 8, 3}; }
 constexpr int kLdsDefaultCb = 1024;
 // Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block
 // widths cover the common cases (K <= 9):

@@ -88,6 +88,27 @@ def ref_gated_dwconv_grads(z, cu_seqlens, weight, bias, dy, compute_dtype=torch.
     return y.detach(), zr.grad, wr.grad, (None if br is None else br.grad)
 
 
+def ref_ln_dwconv_grads(x, cu_seqlens, ln_weight, ln_bias, weight, bias, dy, eps=1e-5, compute_dtype=torch.float64,
+                        residual=False):
+    """(y, dx, d ln_weight, d ln_bias, dw, db) of a conv sub-module in the reference's pre-norm layer
+    (``x + attn(attn_norm(x))``, modeling.py:404-414, the norm a ``torch.nn.LayerNorm`` over the hidden dimension,
+    modeling.py:264-266): ``F.layer_norm`` over the channels, then ``ref_dwconv_varlen``, plus the raw x with
+    ``residual``; gradients by autograd, everything in ``compute_dtype``. With ``dy=None`` only y."""
+    xr = x.detach().to(compute_dtype).requires_grad_(True)
+    gr = ln_weight.detach().to(compute_dtype).requires_grad_(True)
+    hr = None if ln_bias is None else ln_bias.detach().to(compute_dtype).requires_grad_(True)
+    wr = weight.detach().to(compute_dtype).requires_grad_(True)
+    br = None if bias is None else bias.detach().to(compute_dtype).requires_grad_(True)
+    n = F.layer_norm(xr, (xr.shape[1],), gr, hr, eps)
+    y = ref_dwconv_varlen(n, cu_seqlens, wr, br, compute_dtype, False)
+    if residual:
+        y = y + xr
+    if dy is None:
+        return y.detach()
+    y.backward(dy.to(compute_dtype))
+    return (y.detach(), xr.grad, gr.grad, None if hr is None else hr.grad, wr.grad, None if br is None else br.grad)
+
+
 # --------------------------------------------------------------------------------------------
 # C oracle (definition, double accumulation)
 # --------------------------------------------------------------------------------------------

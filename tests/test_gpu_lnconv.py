@@ -1,0 +1,97 @@
+"""LayerNorm fused into the conv's forward (a conv sub-module of the reference's pre-norm layer, modeling.py:404-414)
+against the float64 oracle, through the C ABI entry point and the autograd surface."""
+import pytest
+import torch
+
+import nanoplm_amd as npa
+from nanoplm_amd import _lib
+from nanoplm_amd.workloads import cu_from_lengths, make_workload
+from oracle import dwconv_ref as O
+from tests.gpu_util import assert_act_close, assert_red_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+LENS_MIX = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 17, 512, 23, 24, 25, 47, 48, 49]
+
+
+def _case(lens, C, K, dt, wdt, seed, ln_bias=True):
+    g = torch.Generator().manual_seed(seed)
+    T = int(sum(lens))
+    x = (torch.randn(T, C, generator=g) * (1 + torch.rand(T, 1, generator=g) * 3) + torch.randn(T, 1, generator=g)).to(dt)
+    gam = (1 + 0.3 * torch.randn(C, generator=g)).to(wdt)
+    bet = (0.2 * torch.randn(C, generator=g)).to(wdt) if ln_bias else None
+    w = (torch.randn(C, K, generator=g) * K ** -0.5).to(wdt)
+    b = (torch.randn(C, generator=g) * 0.02).to(wdt)
+    dy = torch.randn(T, C, generator=g).to(dt)
+    return x, cu_from_lengths(torch.tensor(lens)), gam, bet, w, b, dy
+
+
+def _check_fwd(x, cu, gam, bet, w, b, what, residual=False, fused=True):
+    y64 = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, None, 1e-5, torch.float64, residual)
+    xd, cud, gd, wd, bd = (t.to(DEV) for t in (x, cu, gam, w, b))
+    hd = None if bet is None else bet.to(DEV)
+    assert npa.ln_supported(xd, wd) == fused
+    y, stats = npa.ln_dwconv_fwd(xd, cud, gd, hd, wd, bd, residual=residual)
+    assert_act_close(y, y64, x.dtype, what + " y")
+    x64 = x.double()
+    mean = x64.mean(1)
+    rstd = 1 / torch.sqrt(x64.var(1, unbiased=False) + 1e-5)
+    torch.testing.assert_close(stats[:, 0].cpu().double(), mean, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(stats[:, 1].cpu().double(), rstd, rtol=1e-5, atol=1e-6)
+    return y
+
+
+@pytest.mark.parametrize("K", [3, 5, 7, 9])
+@pytest.mark.parametrize("dt,wdt,C", [(torch.bfloat16, torch.bfloat16, 1024), (torch.bfloat16, torch.float32, 768),
+                                       (torch.float32, torch.float32, 512), (torch.float32, torch.float32, 384),
+                                       (torch.bfloat16, torch.bfloat16, 8), (torch.float32, torch.bfloat16, 100)])
+def test_fused_layernorm_forward_kernel_sizes_and_widths(K, dt, wdt, C):
+    """Whole rows in one 2 KiB column block: full and partial rows, one chunk per row, both dtypes, mixed
+    parameter dtypes; lengths around the 24-row tiles and the 12-row wave windows, empty sequences."""
+    print(f"[case] ln K={K} C={C} {dt} w {wdt}", flush=True)
+    _check_fwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C)[:6], f"ln K={K} C={C} {dt}")
+    _check_fwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False)[:6], f"ln residual K={K} C={C} {dt}",
+               residual=True)
+
+
+def test_fused_layernorm_forward_is_deterministic_and_takes_the_boundary_stress_mix():
+    wl = make_workload(5, T=20011, C=1024, with_dy=False)        # lengths of 1..8 mixed with 400..512, odd T
+    g = torch.Generator().manual_seed(5)
+    gam = (1 + 0.3 * torch.randn(1024, generator=g)).bfloat16()
+    bet = (0.2 * torch.randn(1024, generator=g)).bfloat16()
+    y = _check_fwd(wl.x, wl.cu_seqlens, gam, bet, wl.weight, wl.bias, "ln boundary stress", residual=True)
+    a = [t.to(DEV) for t in (wl.x, wl.cu_seqlens, gam, bet, wl.weight, wl.bias)]
+    y2, _ = npa.ln_dwconv_fwd(*a, residual=True)
+    assert torch.equal(y, y2)
+
+
+def test_shapes_outside_the_fused_kernel_compose_layer_norm_and_the_conv():
+    for (C, K, dt) in ((2048, 7, torch.bfloat16), (1024, 7, torch.float32), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
+        print(f"[case] ln composed C={C} K={K} {dt}", flush=True)
+        _check_fwd(*_case([5, 40, 3, 0, 90], C, K, dt, dt, seed=C + K)[:6], f"ln composed C={C} K={K}", residual=True, fused=False)
+
+
+@pytest.mark.parametrize("dt,C,residual", [(torch.bfloat16, 1024, True), (torch.float32, 512, False), (torch.bfloat16, 2048, True)])
+def test_autograd_through_the_fused_forward(dt, C, residual):
+    """Gradients of x, the LayerNorm parameters and the conv parameters against the float64 oracle (the last case
+    is a width the fused kernel does not take: same surface, composed ops)."""
+    x, cu, gam, bet, w, b, dy = _case(LENS_MIX, C, 7, dt, torch.float32, seed=C)
+    y64, dx64, dg64, dh64, dw64, db64 = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, dy, 1e-5, torch.float64, residual)
+    xd = x.to(DEV).requires_grad_(True)
+    params = [t.to(DEV).requires_grad_(True) for t in (gam, bet, w, b)]
+    y = npa.ln_varlen_dwconv(xd, cu.to(DEV), params[0], params[1], params[2], params[3], residual=residual)
+    y.backward(dy.to(DEV))
+    assert_act_close(y.detach(), y64, dt, "y")
+    assert_act_close(xd.grad, dx64, dt, "dx")
+    assert_red_close(params[0].grad, dg64, "d ln_weight")
+    assert_red_close(params[1].grad, dh64, "d ln_bias")
+    assert_red_close(params[2].grad, dw64, "dw")
+    assert_red_close(params[3].grad, db64, "db")
+
+
+def test_unsupported_arguments_are_refused():
+    x, cu, gam, bet, w, b, dy = _case([5, 9], 64, 7, torch.float32, torch.float32, seed=1)
+    with pytest.raises(RuntimeError):
+        npa.ln_dwconv_fwd(x, cu, gam, bet, w, b)                      # CPU tensors
+    with pytest.raises(ValueError):
+        npa.ln_dwconv_fwd(x.to(DEV), cu.to(DEV), gam[:-1].to(DEV), None, w.to(DEV), None)

@@ -342,3 +342,43 @@ def test_gated_oracle_against_closed_forms_and_finite_differences():
     z1[:, C:] = 40.0
     torch.testing.assert_close(O.ref_gated_dwconv_grads(z1, cu, w, b, None), O.ref_dwconv_varlen(40.0 * z[:, :C], cu, w, b, torch.float64),
                                rtol=1e-14, atol=1e-12)
+
+
+def test_layernorm_conv_oracle_against_the_written_out_formula_and_finite_differences():
+    """ref_ln_dwconv_grads (F.layer_norm, then the conv loop, by autograd) against the formula written out -
+    n = (x - mean) / sqrt(var + eps) * gamma + beta with the biased variance of a row, fed to the C restatement -
+    and its gradients against central differences of that forward."""
+    g = torch.Generator().manual_seed(11)
+    lens = [1, 2, 5, 0, 9, 3]
+    T, C, K, eps = sum(lens), 24, 5, 1e-5
+    x = torch.randn(T, C, generator=g, dtype=torch.float64) * 2 + 0.5
+    gam = torch.randn(C, generator=g, dtype=torch.float64)
+    bet = torch.randn(C, generator=g, dtype=torch.float64)
+    w = torch.randn(C, K, generator=g, dtype=torch.float64)
+    b = torch.randn(C, generator=g, dtype=torch.float64)
+    dy = torch.randn(T, C, generator=g, dtype=torch.float64)
+    cu = cu_from_lengths(torch.tensor(lens))
+    for residual in (False, True):
+        y, dx, dgam, dbet, dw, db = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, dy, eps, torch.float64, residual)
+        mean = x.mean(1, keepdim=True)
+        var = ((x - mean) ** 2).mean(1, keepdim=True)
+        n = (x - mean) / torch.sqrt(var + eps) * gam + bet
+        y2 = O.brute_force(n, cu, w, b) + (x if residual else 0)
+        torch.testing.assert_close(y, y2, rtol=1e-12, atol=1e-12)
+
+        def loss(xx, gg, hh):
+            return float((O.ref_ln_dwconv_grads(xx, cu, gg, hh, w, b, None, eps, torch.float64, residual) * dy).sum())
+        h = 1e-6
+        for (t, c) in ((0, 0), (4, 7), (T - 1, C - 1), (9, 3)):
+            e = torch.zeros_like(x); e[t, c] = h
+            fd = (loss(x + e, gam, bet) - loss(x - e, gam, bet)) / (2 * h)
+            assert abs(fd - float(dx[t, c])) < 1e-6 * max(1.0, abs(fd))
+        for c in (0, 5, C - 1):
+            e = torch.zeros_like(gam); e[c] = h
+            fd = (loss(x, gam + e, bet) - loss(x, gam - e, bet)) / (2 * h)
+            assert abs(fd - float(dgam[c])) < 1e-6 * max(1.0, abs(fd))
+            fd = (loss(x, gam, bet + e) - loss(x, gam, bet - e)) / (2 * h)
+            assert abs(fd - float(dbet[c])) < 1e-6 * max(1.0, abs(fd))
+    # without a LayerNorm bias
+    y = O.ref_ln_dwconv_grads(x, cu, gam, None, w, b, None, eps)
+    torch.testing.assert_close(y, O.brute_force((x - mean) / torch.sqrt(var + eps) * gam, cu, w, b), rtol=1e-12, atol=1e-12)
