@@ -147,6 +147,9 @@ def main():
     ap.add_argument("--gated", action="store_true",
                     help="gated variant: input z = [x_proj | gate] of width 2C, conv over x_proj * silu(gate) "
                          "(informational; per-kernel figures then bracket backward + finalize together)")
+    ap.add_argument("--ln", action="store_true",
+                    help="LayerNorm-fused forward: y = x + conv(layer_norm(x)) in one kernel (forward pass only; "
+                         "configurations whose rows fit 2 KiB: 2, 3, 5)")
     ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
     ap.add_argument("--prewarm-ms", type=float, default=1000.0,
                     help="untimed steps run for this long before the warm-up steps")
@@ -171,7 +174,9 @@ def main():
     wl = make_workload(args.config, with_dy=True)
     d = wl.to(dev)
     T, C, K, S = wl.T, wl.C, wl.K, wl.S
-    fwd_bwd = wl.passes == "fwd+bwd"
+    fwd_bwd = wl.passes == "fwd+bwd" and not args.ln
+    if args.ln and (args.gated or C * d.x.element_size() > 2048 or K > 9):
+        sys.exit("--ln needs rows of at most 2 KiB and K <= 9 (configurations 2, 3, 5) and excludes --gated")
     NSET = 4
     BWD_SHIFT = 2          # the backward of step i uses set (i + BWD_SHIFT) % NSET
     if args.gated and not fwd_bwd:
@@ -191,9 +196,18 @@ def main():
     ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     cu, w, b = d.cu_seqlens, d.weight, d.bias
-    flags = _lib.RESIDUAL if args.residual else 0
+    flags = _lib.RESIDUAL if (args.residual or args.ln) else 0
+    if args.ln:
+        ln_w = (1 + 0.1 * torch.randn(C, device=dev)).to(w.dtype)
+        ln_b = (0.1 * torch.randn(C, device=dev)).to(w.dtype)
+        stats = torch.empty((T, 2), dtype=torch.float32, device=dev)
     def fwd(i):
         j = i % NSET
+        if args.ln:
+            _lib.check(lib.nplm_dwconv_ln_fwd(xs[j].data_ptr(), cu.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), 1e-5,
+                                              w.data_ptr(), b.data_ptr(), ys[j].data_ptr(), stats.data_ptr(), T, C, K, S,
+                                              act, act, flags, stream), "nplm_dwconv_ln_fwd")
+            return
         if args.gated:
             _lib.check(lib.nplm_dwconv_gated_fwd(xs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), b.data_ptr(),
                                                  ys[j].data_ptr(), T, C, K, S, act, act, flags, stream), "nplm_dwconv_gated_fwd")
@@ -304,7 +318,7 @@ def main():
     def roof(nbytes, samples_us, kernel):
         med = statistics.median(samples_us)
         gbps = nbytes / med / 1e3
-        traffic = None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel))
+        traffic = None if (args.gated or args.residual or args.ln) else MEASURED_TRAFFIC.get((wl.name, kernel))
         r = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
              "traffic": traffic, "kernel": kernel, "median_us": med, "min_us": min(samples_us),
              "avg_us": statistics.fmean(samples_us), "launches": len(samples_us), "algorithmic_bytes": nbytes}
@@ -315,8 +329,9 @@ def main():
 
     out = {
         "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
-                  if args.config == 3 and not args.gated else
-                  f"varlen {'gated ' if args.gated else ''}dwconv {wl.passes} tokens/s ({wl.name})",
+                  if args.config == 3 and not args.gated and not args.ln else
+                  f"varlen {'gated ' if args.gated else 'layernorm-fused ' if args.ln else ''}dwconv "
+                  f"{'fwd' if args.ln else wl.passes} tokens/s ({wl.name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_min": min(rep_ms), "reps": len(rep_ms),
         "ms_per_step_reps": [round(v, 5) for v in rep_ms], "prewarm_ms": prewarm_ms, "prewarm_steps": prewarm_steps,
@@ -324,8 +339,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
-        "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
-                   "rotating_sets": NSET, "backward_set_shift": BWD_SHIFT if fwd_bwd else None, "residual": bool(args.residual), "gated": bool(args.gated)},
+        "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": "fwd" if args.ln else wl.passes,
+                   "rotating_sets": NSET, "backward_set_shift": BWD_SHIFT if fwd_bwd else None, "residual": bool(args.residual or args.ln), "gated": bool(args.gated), "layernorm": bool(args.ln)},
         "step_algorithmic_bytes": step_bytes,
         "step_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,

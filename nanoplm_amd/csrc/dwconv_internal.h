@@ -196,7 +196,7 @@ constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
 // bytes per lane, 2 row groups of 8 rows (16-row tiles of K + 15 staged rows), 8 compute + 8 loader waves, three tiles
 // (one computed, one having its row statistics taken by the loader waves, one in flight: 132 KiB at K = 7). With two
 // 24-row tiles nothing is in flight while the statistics of a tile are taken, and the forward runs at 148 us instead of
-// 115 - 120 us (T=131072, C=1024, K=7, bf16).
+// 108 us (T=131072, C=1024, K=7, bf16).
 constexpr bool lds_ln_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
 constexpr int kLnCbBytes = 2048;
 constexpr LdsShapeSel lds_ln_shape(bool bf16) { return LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 8, 3}; }
