@@ -148,8 +148,9 @@ def main():
                     help="gated variant: input z = [x_proj | gate] of width 2C, conv over x_proj * silu(gate) "
                          "(informational; per-kernel figures then bracket backward + finalize together)")
     ap.add_argument("--ln", action="store_true",
-                    help="LayerNorm-fused forward: y = x + conv(layer_norm(x)) in one kernel (forward pass only; "
-                         "configurations whose rows fit 2 KiB: 2, 3, 5)")
+                    help="LayerNorm-fused variant: y = x + conv(layer_norm(x)) in one forward kernel; the backward (conv "
+                         "backward over the re-normalised x, then the LayerNorm input gradient) is bracketed as one "
+                         "figure like --gated (configurations whose rows fit 2 KiB: 2, 3, 5)")
     ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
     ap.add_argument("--prewarm-ms", type=float, default=1000.0,
                     help="untimed steps run for this long before the warm-up steps")
@@ -174,7 +175,7 @@ def main():
     wl = make_workload(args.config, with_dy=True)
     d = wl.to(dev)
     T, C, K, S = wl.T, wl.C, wl.K, wl.S
-    fwd_bwd = wl.passes == "fwd+bwd" and not args.ln
+    fwd_bwd = wl.passes == "fwd+bwd"
     if args.ln and (args.gated or C * d.x.element_size() > 2048 or K > 9):
         sys.exit("--ln needs rows of at most 2 KiB and K <= 9 (configurations 2, 3, 5) and excludes --gated")
     NSET = 4
@@ -190,7 +191,8 @@ def main():
     dw = torch.empty((C, K), dtype=torch.float32, device=dev)
     db = torch.empty((C,), dtype=torch.float32, device=dev)
     act = _lib.BF16 if wl.dtype == torch.bfloat16 else _lib.F32
-    ws_bytes = int((lib.nplm_dwconv_gated_bwd_workspace_bytes if args.gated else lib.nplm_dwconv_bwd_workspace_bytes)(T, C, K, act))
+    ws_bytes = int((lib.nplm_dwconv_gated_bwd_workspace_bytes if args.gated else lib.nplm_dwconv_ln_bwd_workspace_bytes if args.ln
+                    else lib.nplm_dwconv_bwd_workspace_bytes)(T, C, K, act))
     if args.gated and ws_bytes == 0:
         sys.exit("the fused gated kernels are not built for this configuration")
     ws = torch.empty((max(ws_bytes, 256),), dtype=torch.uint8, device=dev)
@@ -200,12 +202,13 @@ def main():
     if args.ln:
         ln_w = (1 + 0.1 * torch.randn(C, device=dev)).to(w.dtype)
         ln_b = (0.1 * torch.randn(C, device=dev)).to(w.dtype)
-        stats = torch.empty((T, 2), dtype=torch.float32, device=dev)
+        stats = [torch.empty((T, 2), dtype=torch.float32, device=dev) for _ in range(NSET)]
+        dln = torch.empty((2, C), dtype=torch.float32, device=dev)
     def fwd(i):
         j = i % NSET
         if args.ln:
             _lib.check(lib.nplm_dwconv_ln_fwd(xs[j].data_ptr(), cu.data_ptr(), ln_w.data_ptr(), ln_b.data_ptr(), 1e-5,
-                                              w.data_ptr(), b.data_ptr(), ys[j].data_ptr(), stats.data_ptr(), T, C, K, S,
+                                              w.data_ptr(), b.data_ptr(), ys[j].data_ptr(), stats[j].data_ptr(), T, C, K, S,
                                               act, act, flags, stream), "nplm_dwconv_ln_fwd")
             return
         if args.gated:
@@ -219,7 +222,14 @@ def main():
         j = (i + shift) % NSET
         args_ = (xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(),
                  db.data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act)
-        if args.gated:
+        if args.ln:
+            rc = lib.nplm_dwconv_ln_bwd(xs[j].data_ptr(), gs[j].data_ptr(), cu.data_ptr(), stats[j].data_ptr(), ln_w.data_ptr(),
+                                        ln_b.data_ptr(), w.data_ptr(), dxs[j].data_ptr(), dw.data_ptr(), db.data_ptr(),
+                                        dln[0].data_ptr(), dln[1].data_ptr(), ws.data_ptr(), ws.numel(), T, C, K, S, act, act,
+                                        flags, stream)
+            if t is not None and t.mid_event:      # no mid-call event on this entry point: mark the end instead
+                HipEvents.record_raw(t.mid_event, stream)
+        elif args.gated:
             rc = lib.nplm_dwconv_gated_bwd(*args_, flags, stream)
             if t is not None and t.mid_event:      # no mid-call event on this entry point: mark the end instead
                 HipEvents.record_raw(t.mid_event, stream)
@@ -331,7 +341,7 @@ def main():
         "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
                   if args.config == 3 and not args.gated and not args.ln else
                   f"varlen {'gated ' if args.gated else 'layernorm-fused ' if args.ln else ''}dwconv "
-                  f"{'fwd' if args.ln else wl.passes} tokens/s ({wl.name})",
+                  f"{wl.passes} tokens/s ({wl.name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_min": min(rep_ms), "reps": len(rep_ms),
         "ms_per_step_reps": [round(v, 5) for v in rep_ms], "prewarm_ms": prewarm_ms, "prewarm_steps": prewarm_steps,
@@ -339,7 +349,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
         "data": "synthetic (seeded: lengths, x, weight, bias, dy drawn on the CPU, see nanoplm_amd/workloads.py)",
-        "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": "fwd" if args.ln else wl.passes,
+        "config": {"workload": wl.name, "T": T, "C": C, "K": K, "S": S, "passes": wl.passes,
                    "rotating_sets": NSET, "backward_set_shift": BWD_SHIFT if fwd_bwd else None, "residual": bool(args.residual or args.ln), "gated": bool(args.gated), "layernorm": bool(args.ln)},
         "step_algorithmic_bytes": step_bytes,
         "step_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,

@@ -190,6 +190,26 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
                        int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
 
 /*
+ * Backward of nplm_dwconv_ln_fwd (same shapes, same -NPLM_DWCONV_EUNSUPPORTED rule; the reference would reach it
+ * through autograd over torch.nn.LayerNorm, modeling.py:264-266, followed by the conv's backward,
+ * modeling.py:1246-1339). From x, the row statistics the forward wrote and dy:
+ *   dw, db                  the conv's parameter gradients over n = layer_norm(x) (n is recomputed, never stored)
+ *   dln_weight, dln_bias    the LayerNorm's parameter gradients, fp32 [C] (dln_bias may be NULL)
+ *   dx                      the LayerNorm's input gradient (+ dy with NPLM_DWCONV_RESIDUAL), act_dtype
+ * Two kernels and two small reductions: the conv backward that normalises x as it reads and also sums the
+ * LayerNorm parameter gradients, writing dn (the gradient of n, fp32) into the workspace; the reductions of the
+ * per-block partial sums; one pass over (x, dn, dy) rows for dx. The workspace (nplm_dwconv_ln_bwd_workspace_bytes,
+ * 256-byte aligned; 0 for unsupported shapes) holds the partial sums and dn (T x C x 4 bytes).
+ */
+size_t nplm_dwconv_ln_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype);
+int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const float* stats,
+                       const void* ln_weight, const void* ln_bias, const void* w,
+                       void* dx, float* dw, float* db, float* dln_weight, float* dln_bias,
+                       void* workspace, size_t workspace_bytes,
+                       int64_t T, int32_t C, int32_t K, int32_t S,
+                       int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream);
+
+/*
  * Debug helper: copies cu to the host (synchronises `stream`) and verifies the preconditions.
  * Returns 0, -NPLM_DWCONV_ECU, another argument error, or a hipError_t.
  */

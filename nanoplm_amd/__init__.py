@@ -29,6 +29,7 @@ from .gated import (  # noqa: F401
 )
 from .lnconv import (  # noqa: F401
     LnVarlenDWConv1dFunction,
+    ln_dwconv_bwd,
     ln_dwconv_fwd,
     ln_supported,
     ln_varlen_dwconv,

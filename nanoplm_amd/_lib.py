@@ -32,6 +32,8 @@ PUBLIC_SYMBOLS = (
     "nplm_dwconv_gated_bwd_workspace_bytes",
     "nplm_dwconv_gated_bwd",
     "nplm_dwconv_ln_fwd",
+    "nplm_dwconv_ln_bwd_workspace_bytes",
+    "nplm_dwconv_ln_bwd",
     "nplm_dwconv_check_cu",
 )
 
@@ -82,6 +84,10 @@ def load():
     lib.nplm_dwconv_ln_fwd.argtypes = [vp, vp, vp, vp, ctypes.c_float, vp, vp, vp, vp, i64, i32, i32, i32, i32, i32,
                                        ctypes.c_uint32, vp]
     lib.nplm_dwconv_ln_fwd.restype = ctypes.c_int
+    lib.nplm_dwconv_ln_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
+    lib.nplm_dwconv_ln_bwd_workspace_bytes.restype = sz
+    lib.nplm_dwconv_ln_bwd.argtypes = [vp] * 13 + [sz, i64, i32, i32, i32, i32, i32, ctypes.c_uint32, vp]
+    lib.nplm_dwconv_ln_bwd.restype = ctypes.c_int
     lib.nplm_dwconv_gated_bwd_workspace_bytes.argtypes = [i64, i32, i32, i32]
     lib.nplm_dwconv_gated_bwd_workspace_bytes.restype = sz
     lib.nplm_dwconv_gated_bwd.argtypes = bwd_args[:-1] + [ctypes.c_uint32, vp]

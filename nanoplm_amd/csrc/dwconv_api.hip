@@ -676,6 +676,109 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     return -NPLM_DWCONV_EUNSUPPORTED;
 }
 
+// ---- backward of the LayerNorm-fused forward: conv backward over the re-normalised x (NORM variant of
+// dwconv_bwd_lds_kernel: dn, dw, db and the LayerNorm parameter sums), then the LayerNorm input gradient ---------------
+namespace {
+bool ln_supported(bool bf16, int C, int K, uintptr_t align_bits) {
+    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
+    return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
+}
+// workspace: [conv slabs: nbt x (K+1) x C][LayerNorm slabs: nbt x 2 x C][dn: T x C fp32], each part 256-byte aligned
+struct LnBwdLayout {
+    LdsPlan lp;
+    size_t conv_slabs, ln_slabs, dn, total;
+};
+int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
+    nplm_dwconv_tuning t{};
+    const LdsShapeSel sh = lds_default_shape(true, bf16, K);
+    t.vec = sh.vec; t.unroll = sh.rw; t.bt = sh.nrg; t.bw = sh.ncw; t.nwl = sh.nwl;
+    LnBwdLayout l{};
+    int rc = make_lds_plan(true, bf16, T, C, K, &t, &l.lp);
+    if (rc) return rc;
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    l.conv_slabs = up((size_t)l.lp.nbt * (K + 1) * C * sizeof(float));
+    l.ln_slabs = up((size_t)l.lp.nbt * 2 * C * sizeof(float));
+    l.dn = up((size_t)T * C * sizeof(float));
+    l.total = l.conv_slabs + l.ln_slabs + l.dn;
+    *out = l;
+    return 0;
+}
+}  // namespace
+
+size_t nplm_dwconv_ln_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
+    if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    if (!ln_supported(bf16, C, K, 0)) return 0;
+    LnBwdLayout l;
+    if (ln_bwd_layout(bf16, T, C, K, &l)) return 0;
+    return l.total;
+}
+
+int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const float* stats, const void* ln_weight,
+                       const void* ln_bias, const void* w, void* dx, float* dw, float* db, float* dln_weight,
+                       float* dln_bias, void* workspace, size_t workspace_bytes, int64_t T, int32_t C, int32_t K,
+                       int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
+    int rc = check_common(T, C, K, S, act_dtype, w_dtype);
+    if (rc) return rc;
+    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    hipStream_t s = (hipStream_t)stream;
+    if (!dw || !db || !dln_weight) return -NPLM_DWCONV_ENULL;
+    if (T == 0) {
+        hipError_t e = fill_zero(dw, (long long)C * K, s);
+        if (e == hipSuccess) e = fill_zero(db, C, s);
+        if (e == hipSuccess) e = fill_zero(dln_weight, C, s);
+        if (e == hipSuccess) e = fill_zero(dln_bias, C, s);
+        return (int)e;
+    }
+    if (!x || !dy || !cu || !stats || !ln_weight || !w || !dx) return -NPLM_DWCONV_ENULL;
+    const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
+    const uintptr_t E = bf16 ? 2 : 4;
+    const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
+    if (((uintptr_t)w | (uintptr_t)ln_weight | (uintptr_t)ln_bias) % WE || ((uintptr_t)cu | (uintptr_t)stats) % 4 ||
+        ((uintptr_t)dw | (uintptr_t)db | (uintptr_t)dln_weight | (uintptr_t)dln_bias) % 4 ||
+        ((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) % E)
+        return -NPLM_DWCONV_EALIGN;
+    if (!ln_supported(bf16, C, K, (uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx)) return -NPLM_DWCONV_EUNSUPPORTED;
+    LnBwdLayout l;
+    rc = ln_bwd_layout(bf16, T, C, K, &l);
+    if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
+    if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < l.total) return -NPLM_DWCONV_EWORKSPACE;
+    char* ws = reinterpret_cast<char*>(workspace);
+    float* part = reinterpret_cast<float*>(ws);
+    float* part_ln = reinterpret_cast<float*>(ws + l.conv_slabs);
+    float* dn = reinterpret_cast<float*>(ws + l.conv_slabs + l.ln_slabs);
+    // the conv's own residual flag stays off: the identity branch bypasses the LayerNorm and joins in the last kernel
+    const int w_flags = kernel_w_flags(w_dtype, 0);
+    const ConvPtrs la{x, dy, cu, w, nullptr, (void*)dn, part};
+    const LnBwdArgs ln{stats, ln_weight, ln_bias, part_ln};
+    const LdsGeo g = make_lds_geo(l.lp, T, C, S, w_flags);
+    const dim3 grid(l.lp.ncb * l.lp.nbt);
+    hipError_t e = hipErrorInvalidConfiguration;
+    switch (K) {
+        case 3: e = launch_ln_bwd_k3(bf16, la, ln, g, grid, s); break;
+        case 5: e = launch_ln_bwd_k5(bf16, la, ln, g, grid, s); break;
+        case 7: e = launch_ln_bwd_k7(bf16, la, ln, g, grid, s); break;
+        case 9: e = launch_ln_bwd_k9(bf16, la, ln, g, grid, s); break;
+    }
+    if (e != hipSuccess) return (int)e;
+    long long n_out = (long long)(K + 1) * C;
+    hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                       (const float*)part, l.lp.nbt, C, K, dw, db);
+    n_out = 2LL * C;      // the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
+    hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                       (const float*)part_ln, l.lp.nbt, C, 1, dln_weight, dln_bias);
+    int blocks = ceil_div(T, 4);
+    if (blocks > kNumCU * 8) blocks = kNumCU * 8;
+    const void* res = (flags & NPLM_DWCONV_RESIDUAL) ? dy : nullptr;
+    if (bf16)
+        hipLaunchKernelGGL(ln_bwd_dx_kernel<true>, dim3(blocks), dim3(256), 0, s, x, stats, ln_weight, w_flags, (const float*)dn, res,
+                           dx, (int)T, C);
+    else
+        hipLaunchKernelGGL(ln_bwd_dx_kernel<false>, dim3(blocks), dim3(256), 0, s, x, stats, ln_weight, w_flags, (const float*)dn, res,
+                           dx, (int)T, C);
+    return (int)hipGetLastError();
+}
+
 size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;

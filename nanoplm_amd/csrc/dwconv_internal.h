@@ -25,7 +25,7 @@ typedef struct nplm_dwconv_tuning {
     int32_t xcd_remap;  // 1 = give each XCD a contiguous share of the token-blocks (off by default: measured slower)
     int32_t maxt;       // launch-bounds class (threads per block the kernel was compiled for)
     int32_t algo;       // 1 = sliding-window (register) kernels, 2 = LDS-staged pipelined kernels,
-                        // 3 = role-split LDS-staged backward (K = 31)
+                        // 3 = role-split LDS-staged kernels (K = 31, 15)
     int32_t nwl;        // LDS kernels: loader waves per block
     int32_t nbuf;       // LDS forward: tile buffers (2 or 3)
     uint32_t flags;     // NPLM_DWCONV_RESIDUAL etc., as for the _ex entry points
@@ -114,7 +114,7 @@ hipError_t launch_bwd_gated_k31(bool bf16, int unroll, int maxt, const ConvPtrs&
 // and LDS-staged forward with the gate formed in LDS by the loader waves
 hipError_t launch_fwd_lds_gated_k15(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
-// role-split LDS kernels at K = 31 (fixed shape per dtype, see lds_split_shape())
+// role-split LDS kernels at K = 31 and 15 (fixed shape per dtype, see lds_split_shape())
 hipError_t launch_bwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_bwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
@@ -123,6 +123,11 @@ hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+// conv backward over layer_norm(x) (the NORM variant of dwconv_bwd_lds_kernel on the default backward shape)
+hipError_t launch_ln_bwd_k3(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k5(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k7(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k9(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)

@@ -577,10 +577,24 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 // a buffer holds the dy tile, a u tile and a g tile; h rows (for dw) and the two halves of dz
 //     du = dh * silu(g),   dg = dh * u * sig(g) * (1 + g * (1 - sig(g))),   dh = the conv's dx
 // are formed in registers from the staged u and g rows.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false>
+//
+// NORM: the conv ran over n = layer_norm(x; gamma, beta) (statistics per row in `stats`, see dwconv_ln_kernels.h) and x is
+// the raw input: the wave normalises its x rows as it reads them, dx is the gradient with respect to n, and the
+// block also sums the LayerNorm parameter gradients, which need that gradient in fp32 and the normalised rows:
+//     dgamma[c] += dn[t,c] * xhat[t,c],   dbeta[c] += dn[t,c],   xhat = (x - mean) * rstd.
+// They leave the block like dw/db, in a second slab of 2 x C floats per token block.
+struct LnBwdArgs {
+    const float* stats;    // [T][2] fp32 (mean, rstd)
+    const void* gamma;     // [C], weight dtype
+    const void* beta;      // [C] or null
+    float* partial2;       // [nbt][2][C]: dgamma, dbeta partial sums
+};
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false, bool NORM = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
-                      const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g) {
+                      const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g,
+                      const LnBwdArgs ln) {
+    static_assert(!NORM || (WDX && WDW && !GATED), "the LayerNorm variant produces every gradient of the plain conv");
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     constexpr int XT_BYTES = R * SH::CB_BYTES;
@@ -632,11 +646,22 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     float wr[VEC][K];
     float dwa[VEC][K];
     float dba[VEC];
+    float dga[NORM ? VEC : 1], dbb[NORM ? VEC : 1], gam[NORM ? VEC : 1], bet[NORM ? VEC : 1];   // LayerNorm: sums and parameters
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
         dba[v] = 0.f;
 #pragma unroll
         for (int k = 0; k < K; ++k) { dwa[v][k] = 0.f; wr[v][k] = 0.f; }
+    }
+    if constexpr (NORM) {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            const bool wb = (g.w_flags & W_BF16) != 0;
+            dga[v] = 0.f; dbb[v] = 0.f;
+            const int c = c0 + v < C ? c0 + v : C - 1;
+            gam[v] = wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.gamma)[c]) : reinterpret_cast<const float*>(ln.gamma)[c];
+            bet[v] = !ln.beta ? 0.f : wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.beta)[c]) : reinterpret_cast<const float*>(ln.beta)[c];
+        }
     }
     if (is_loader) {
         stage_both(lds_raw, tb * R);
@@ -669,6 +694,17 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
                 const char* lpx = cur + SH::TILE_BYTES + loff;     // x : staged row u <-> global row tf + u
                 const rsrc_t ro = rows_rsrc(dx, tf, T, x_row_bytes);
+                // LayerNorm: (rstd, -mean * rstd) of the wave's x rows, wave-uniform
+                float sa[NORM ? RW : 1], sb[NORM ? RW : 1];
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) {
+                        const int tr = tf + u < T ? tf + u : T - 1;
+                        const float mean = ln.stats[2 * (size_t)tr], rstd = ln.stats[2 * (size_t)tr + 1];
+                        sa[u] = rstd;
+                        sb[u] = -mean * rstd;
+                    }
+                }
                 // Gated: per element of the wave's x rows, the two factors everything else needs:
                 //   gs = silu(g) / ... = g * sig(g)              (h = u * gs, du = dh * gs)
                 //   gd = u * sig(g) * (1 + g * (1 - sig(g)))     (dg = dh * gd)
@@ -688,6 +724,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         }
                     } else {
                         lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                        if constexpr (NORM) {
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) xv[v] = __builtin_fmaf(__builtin_fmaf(xv[v], sa[u], sb[u]), gam[v], bet[v]);
+                        }
                     }
                 };
                 // write the wave's dx rows (du and dg rows of dz when gated) from the conv's input gradient
@@ -712,13 +752,43 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                 }
                             }
                         } else {
-                            Row o[RW];
+                            if constexpr (NORM) {
+                                // the LayerNorm parameter gradients from the fp32 gradient of n and the normalised row
 #pragma unroll
-                            for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
-                            if (active) {
+                                for (int u = 0; u < RW; ++u) {
+                                    if (tf + u < T) {
+                                        float xr[VEC];
+                                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
 #pragma unroll
-                                for (int u = 0; u < RW; ++u)
-                                    if (tf + u < T) o[u].bstore(ro, out_voff, u * xrowb);
+                                        for (int v = 0; v < VEC; ++v) {
+                                            dga[v] = __builtin_fmaf(acc[u][v], __builtin_fmaf(xr[v], sa[u], sb[u]), dga[v]);
+                                            dbb[v] += acc[u][v];
+                                        }
+                                    }
+                                }
+                            }
+                            if constexpr (NORM) {
+                                // the gradient of n leaves in fp32 whatever the activations are: the row pass that
+                                // turns it into dx rounds once
+                                const int nrowb = C * 4;
+                                const rsrc_t rn = rows_rsrc(dx, tf, T, (size_t)nrowb);
+                                RowVec<false, VEC> o[RW];
+#pragma unroll
+                                for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                                if (active) {
+#pragma unroll
+                                    for (int u = 0; u < RW; ++u)
+                                        if (tf + u < T) o[u].bstore(rn, c0 * 4, u * nrowb);
+                                }
+                            } else {
+                                Row o[RW];
+#pragma unroll
+                                for (int u = 0; u < RW; ++u) o[u].from_f32(acc[u]);
+                                if (active) {
+#pragma unroll
+                                    for (int u = 0; u < RW; ++u)
+                                        if (tf + u < T) o[u].bstore(ro, out_voff, u * xrowb);
+                                }
                             }
                         }
                     }
@@ -842,6 +912,11 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) dst[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : dba[v];
             }
+            if constexpr (NORM) {
+                float* dst = ln.partial2 + (size_t)tb * 2 * C + c0;
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) { dst[v] = dga[v]; dst[C + v] = dbb[v]; }
+            }
         }
         return;
     }
@@ -849,10 +924,11 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     // (the tiles are dead after the last barrier above; loader waves only keep the barriers company)
     float* red = reinterpret_cast<float*>(lds_raw);   // [NWC][VEC][64]
 #pragma unroll
-    for (int kk = 0; kk <= K; ++kk) {
+    for (int kk = 0; kk <= K + (NORM ? 2 : 0); ++kk) {
         float val[VEC];
 #pragma unroll
-        for (int v = 0; v < VEC; ++v) val[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : dba[v];
+        for (int v = 0; v < VEC; ++v)
+            val[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : (kk == K) ? dba[v] : (kk == K + 1) ? dga[NORM ? v : 0] : dbb[NORM ? v : 0];
         if (!is_loader && rg > 0) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v) red[(wv * VEC + v) * 64 + lane] = val[v];
@@ -866,7 +942,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
             }
             if (active) {
-                float* dst = slab + (size_t)kk * C + c0;
+                float* dst = kk <= K ? slab + (size_t)kk * C + c0 : ln.partial2 + ((size_t)tb * 2 + (kk - K - 1)) * C + c0;
 #pragma unroll
                 for (int v = 0; v < VEC; ++v) dst[v] = val[v];
             }

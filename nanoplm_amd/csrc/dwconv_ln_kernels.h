@@ -425,4 +425,94 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// LayerNorm backward with respect to its input, given the gradient dn of the normalised tensor (fp32: what the NORM
+// variant of dwconv_bwd_lds_kernel writes as dx) and the row statistics of the forward:
+//     g = gamma * dn,   dx = rstd * (g - mean_c(g) - xhat * mean_c(g * xhat))  (+ dy: the residual connection's share)
+// The parameter gradients are summed by the conv backward, where dn is still in fp32. One wave per row (rows of at
+// most 2 KiB: two 16-byte chunks per lane), 4 rows per block, blocks stride over the rows; four streams of [T, C].
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_allsum(float v) {
+    v += dpp_row_ror<8>(v);
+    v += dpp_row_ror<4>(v);
+    v += dpp_row_ror<2>(v);
+    v += dpp_row_ror<1>(v);
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return (a + b) + (c + d);
+}
+
+template <bool BF16>
+__global__ void __launch_bounds__(256)
+ln_bwd_dx_kernel(const void* __restrict__ x, const float* __restrict__ stats, const void* __restrict__ gamma, int w_flags,
+                 const float* __restrict__ dn, const void* __restrict__ dy, void* __restrict__ dx, int T, int C) {
+    constexpr int E = BF16 ? 2 : 4, CE = 16 / E, NCH = 2;
+    using Chunk = RowVec<BF16, CE>;
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    const int rowb = C * E;
+    const float inv_c = 1.f / (float)C;
+    float gam[NCH][CE];
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+#pragma unroll
+        for (int e = 0; e < CE; ++e) {
+            const int c = (lane + 64 * i) * CE + e;
+            gam[i][e] = c >= C ? 0.f : (w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(gamma)[c])
+                                                       : reinterpret_cast<const float*>(gamma)[c];
+        }
+    }
+    for (int t = (int)blockIdx.x * 4 + wv; t < T; t += (int)gridDim.x * 4) {
+        const float mean = stats[2 * (size_t)t], rstd = stats[2 * (size_t)t + 1];
+        const float sb = -mean * rstd;
+        const size_t row = (size_t)t * rowb;
+        float gv[NCH][CE], xh[NCH][CE], res[NCH][CE];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int off = (lane + 64 * i) * 16;
+            if (off < rowb) {
+                Chunk cx;
+                float xv[CE], dv[CE];
+                cx.load(reinterpret_cast<const char*>(x) + row + off);
+                cx.to_f32(xv);
+                const float4* gp = reinterpret_cast<const float4*>(dn + (size_t)t * C + (lane + 64 * i) * CE);
+#pragma unroll
+                for (int e = 0; e < CE; e += 4) {
+                    const float4 q = gp[e / 4];
+                    dv[e] = q.x; dv[e + 1] = q.y; dv[e + 2] = q.z; dv[e + 3] = q.w;
+                }
+                if (dy) {
+                    Chunk cr;
+                    cr.load(reinterpret_cast<const char*>(dy) + row + off);
+                    cr.to_f32(res[i]);
+                }
+#pragma unroll
+                for (int e = 0; e < CE; ++e) {
+                    if (!dy) res[i][e] = 0.f;
+                    xh[i][e] = __builtin_fmaf(xv[e], rstd, sb);
+                    gv[i][e] = gam[i][e] * dv[e];
+                    s1 += gv[i][e];
+                    s2 = __builtin_fmaf(gv[i][e], xh[i][e], s2);
+                }
+            }
+        }
+        const float m1 = wave_allsum(s1) * inv_c, m2 = wave_allsum(s2) * inv_c;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int off = (lane + 64 * i) * 16;
+            if (off < rowb) {
+                float o[CE];
+#pragma unroll
+                for (int e = 0; e < CE; ++e) o[e] = __builtin_fmaf(rstd, gv[i][e] - m1 - xh[i][e] * m2, res[i][e]);
+                Chunk co;
+                co.from_f32(o);
+                co.store(reinterpret_cast<char*>(dx) + row + off);
+            }
+        }
+    }
+}
+
 }  // namespace nplm

@@ -9,10 +9,10 @@ For a conv that takes the place of a sub-module of the reference's pre-norm enco
 ``x + conv(layer_norm(x))`` from one read of x and one write of y: the kernel's blocks own whole rows (rows of at
 most 2 KiB: C <= 1024 in bf16, 512 in fp32; K in {3,5,7,9}), take the row statistics from the tile they have staged
 and normalise as they read. The normalised tensor is never stored; the kernel leaves (mean, rstd) per row for the
-backward, which recomputes it: the backward is a composition (normalise with elementwise ops in fp32, this library's
-conv backward, ATen's LayerNorm backward), so the fusion saves forward traffic and the activation memory of the
-normalised tensor, not backward traffic. Shapes the fused kernel is not built for (the library says so with its
-return code) run ``F.layer_norm`` and the plain HIP conv.
+backward, whose conv kernel normalises x again as it reads it, sums the LayerNorm parameter gradients beside dw and db
+and hands the gradient of the normalised tensor to one more pass over the rows for dx. Shapes the fused kernels are
+not built for (the library says so with its return code) compose elementwise normalisation, the plain HIP conv and
+ATen's LayerNorm backward.
 """
 from __future__ import annotations
 
@@ -77,9 +77,61 @@ def ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: 
     return y, stats
 
 
+def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, residual: bool = False):
+    """Raw backward of :func:`ln_dwconv_fwd`: ``(dx, dln_weight, dln_bias, dw, db)``; dx in x's dtype, the rest fp32
+    (dln_bias None without ``ln_bias``). ``stats`` is the forward's ``[T, 2]`` (mean, rstd).
+
+    Fused shapes: the conv backward normalises x as it reads it (the normalised tensor is never stored) and sums the
+    LayerNorm parameter gradients beside dw and db; one more pass over (x, dn, dy) gives dx. Other shapes compose
+    elementwise normalisation in fp32, the plain HIP conv backward and ATen's LayerNorm backward."""
+    T, C, K, S = _check(x, cu_seqlens, ln_weight, ln_bias, weight, None)
+    if dy.shape != x.shape or dy.dtype != x.dtype or dy.device != x.device:
+        raise ValueError("dy must match x in shape, dtype and device")
+    if stats is None or tuple(stats.shape) != (T, 2) or stats.dtype != torch.float32:
+        raise ValueError(f"stats must be the forward's [T={T}, 2] fp32 (mean, rstd)")
+    lib = _lib.load()
+    x = x.contiguous()
+    dy = dy.contiguous()
+    stats = stats.contiguous()
+    weight = weight.contiguous()
+    wdt = weight.dtype
+    lnw = ln_weight.to(wdt).contiguous()
+    lnb = None if ln_bias is None else ln_bias.to(wdt).contiguous()
+    act = _DTYPES[x.dtype]
+    nbytes = int(lib.nplm_dwconv_ln_bwd_workspace_bytes(T, C, K, act)) if T > 0 else 0
+    if nbytes > 0 or T == 0:
+        dx = torch.empty_like(x)
+        dw = torch.empty((C, K), dtype=torch.float32, device=x.device)
+        db = torch.empty((C,), dtype=torch.float32, device=x.device)
+        dg = torch.empty((C,), dtype=torch.float32, device=x.device)
+        dbeta = None if ln_bias is None else torch.empty((C,), dtype=torch.float32, device=x.device)
+        with _launch_on(x) as dev:
+            workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
+            rc = lib.nplm_dwconv_ln_bwd(_ptr(x), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(stats), _ptr(lnw), _ptr(lnb),
+                                        _ptr(weight), _ptr(dx), _ptr(dw), _ptr(db), _ptr(dg), _ptr(dbeta), _ptr(workspace),
+                                        workspace.numel(), T, C, K, S, act, _DTYPES[wdt],
+                                        _lib.RESIDUAL if residual else 0, dev.stream)
+        if rc != -_lib.EUNSUPPORTED:
+            _lib.check(rc, "nplm_dwconv_ln_bwd")
+            return dx, dg, dbeta, dw, db
+    mean, rstd = stats[:, 0:1].contiguous(), stats[:, 1:2].contiguous()     # ATen reads them as dense [T, 1]
+    xf = x.float()
+    gf = lnw.float()
+    n = (xf - mean) * rstd * gf
+    if lnb is not None:
+        n = n + lnb.float()
+    dyf = dy.float()
+    dn, dw, db = varlen_dwconv_bwd(n, dyf, cu_seqlens, weight)
+    dx, dg, dbeta = torch.ops.aten.native_layer_norm_backward(dn, xf, [C], mean, rstd, gf, None if lnb is None else lnb.float(),
+                                                              [True, True, lnb is not None])
+    if residual:
+        dx = dx + dyf
+    return dx.to(x.dtype), dg, (dbeta if lnb is not None else None), dw, db
+
+
 class LnVarlenDWConv1dFunction(torch.autograd.Function):
-    """y = conv(layer_norm(x; ln_weight, ln_bias); weight, bias) (+ x). Forward fused; backward composed (see the
-    module docstring): gradients for x, ln_weight, ln_bias, weight, bias."""
+    """y = conv(layer_norm(x; ln_weight, ln_bias); weight, bias) (+ x): gradients for x, ln_weight, ln_bias, weight,
+    bias. Forward and backward fused where the library has the kernels (see the module docstring)."""
 
     @staticmethod
     def forward(ctx, x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps, residual):
@@ -93,21 +145,10 @@ class LnVarlenDWConv1dFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, cu, ln_weight, ln_bias, weight, stats = ctx.saved_tensors
-        C = x.shape[1]
-        mean, rstd = stats[:, 0:1].contiguous(), stats[:, 1:2].contiguous()     # ATen reads them as dense [T, 1]
-        xf = x.float()
-        gf = ln_weight.float()
-        n = (xf - mean) * rstd * gf
-        if ln_bias is not None:
-            n = n + ln_bias.float()
-        dyf = dy.float().contiguous()
-        dn, dw, db = varlen_dwconv_bwd(n, dyf, cu, weight)
-        bf = None if ln_bias is None else ln_bias.float()
-        dx, dg, dbeta = torch.ops.aten.native_layer_norm_backward(dn, xf, [C], mean, rstd, gf, bf,
-                                                                  [True, True, ln_bias is not None])
-        if ctx.residual:
-            dx = dx + dyf
-        return (dx.to(x.dtype), None, dg.to(ln_weight.dtype), None if ln_bias is None else dbeta.to(ln_bias.dtype),
+        if dy.dtype != x.dtype:
+            dy = dy.to(x.dtype)
+        dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu, stats, ln_weight, ln_bias, weight, residual=ctx.residual)
+        return (dx, None, dg.to(ln_weight.dtype), None if ln_bias is None else dbeta.to(ln_bias.dtype),
                 dw.to(weight.dtype), db.to(ctx.bias_dtype) if ctx.has_bias else None, None, None)
 
 

@@ -1,5 +1,5 @@
-"""LayerNorm fused into the conv's forward (a conv sub-module of the reference's pre-norm layer, modeling.py:404-414)
-against the float64 oracle, through the C ABI entry point and the autograd surface."""
+"""LayerNorm fused into the conv's forward and backward (a conv sub-module of the reference's pre-norm layer,
+modeling.py:404-414) against the float64 oracle, through the C ABI entry points and the autograd surface."""
 import pytest
 import torch
 
@@ -72,9 +72,9 @@ def test_shapes_outside_the_fused_kernel_compose_layer_norm_and_the_conv():
 
 
 @pytest.mark.parametrize("dt,C,residual", [(torch.bfloat16, 1024, True), (torch.float32, 512, False), (torch.bfloat16, 2048, True)])
-def test_autograd_through_the_fused_forward(dt, C, residual):
+def test_autograd_through_the_fused_kernels(dt, C, residual):
     """Gradients of x, the LayerNorm parameters and the conv parameters against the float64 oracle (the last case
-    is a width the fused kernel does not take: same surface, composed ops)."""
+    is a width the fused kernels do not take: same surface, composed ops)."""
     x, cu, gam, bet, w, b, dy = _case(LENS_MIX, C, 7, dt, torch.float32, seed=C)
     y64, dx64, dg64, dh64, dw64, db64 = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, dy, 1e-5, torch.float64, residual)
     xd = x.to(DEV).requires_grad_(True)
@@ -87,6 +87,77 @@ def test_autograd_through_the_fused_forward(dt, C, residual):
     assert_red_close(params[1].grad, dh64, "d ln_bias")
     assert_red_close(params[2].grad, dw64, "dw")
     assert_red_close(params[3].grad, db64, "db")
+
+
+def _check_bwd(x, cu, gam, bet, w, b, dy, what, residual=False, fused=True):
+    _, dx64, dg64, dh64, dw64, db64 = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, dy, 1e-5, torch.float64, residual)
+    xd, cud, gd, wd, dyd = (t.to(DEV) for t in (x, cu, gam, w, dy))
+    hd = None if bet is None else bet.to(DEV)
+    T, C = x.shape
+    ws = _lib.load().nplm_dwconv_ln_bwd_workspace_bytes(T, C, w.shape[1], 1 if x.dtype == torch.bfloat16 else 0)
+    assert (ws > 0) == fused, f"{what}: workspace {ws}"
+    _, stats = npa.ln_dwconv_fwd(xd, cud, gd, hd, wd, None, residual=residual)
+    out = npa.ln_dwconv_bwd(xd, dyd, cud, stats, gd, hd, wd, residual=residual)
+    dx, dg, dh, dw, db = out
+    assert_act_close(dx, dx64, x.dtype, what + " dx")
+    assert_red_close(dg.cpu(), dg64, what + " d ln_weight")
+    assert_red_close(dw.cpu(), dw64, what + " dw")
+    assert_red_close(db.cpu(), db64, what + " db")
+    if bet is None:
+        assert dh is None
+    else:
+        assert_red_close(dh.cpu(), dh64, what + " d ln_bias")
+    return out
+
+
+@pytest.mark.parametrize("K", [3, 5, 7, 9])
+@pytest.mark.parametrize("dt,wdt,C", [(torch.bfloat16, torch.bfloat16, 1024), (torch.bfloat16, torch.float32, 768),
+                                       (torch.float32, torch.float32, 512), (torch.float32, torch.float32, 384),
+                                       (torch.bfloat16, torch.bfloat16, 8), (torch.float32, torch.bfloat16, 100)])
+def test_fused_layernorm_backward_kernel_sizes_and_widths(K, dt, wdt, C):
+    """The conv backward that normalises x as it reads, with the LayerNorm parameter sums, and the row pass for dx:
+    rows of one and two column blocks, partly filled ones, both dtypes, mixed parameter dtypes, with and without the
+    LayerNorm bias and the residual connection; lengths around the 30-row tiles and 10-row wave windows."""
+    print(f"[case] ln bwd K={K} C={C} {dt} w {wdt}", flush=True)
+    _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd K={K} C={C} {dt}")
+    _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd residual K={K} C={C} {dt}",
+               residual=True)
+
+
+def test_fused_layernorm_backward_is_deterministic_and_takes_the_boundary_stress_mix():
+    wl = make_workload(5, T=20011, C=1024, with_dy=True)        # lengths of 1..8 mixed with 400..512, odd T
+    g = torch.Generator().manual_seed(6)
+    gam = (1 + 0.3 * torch.randn(1024, generator=g)).bfloat16()
+    bet = (0.2 * torch.randn(1024, generator=g)).bfloat16()
+    a = (wl.x, wl.cu_seqlens, gam, bet, wl.weight, wl.bias, wl.dy)
+    o1 = _check_bwd(*a, "ln bwd boundary stress", residual=True)
+    o2 = _check_bwd(*a, "ln bwd boundary stress again", residual=True)
+    for p, q in zip(o1, o2):
+        assert torch.equal(p, q)
+
+
+def test_backward_of_shapes_outside_the_fused_kernels_is_composed():
+    for (C, K, dt) in ((2048, 7, torch.bfloat16), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
+        print(f"[case] ln bwd composed C={C} K={K} {dt}", flush=True)
+        _check_bwd(*_case([5, 40, 3, 0, 90], C, K, dt, dt, seed=C + K), f"ln bwd composed C={C} K={K}", residual=True, fused=False)
+
+
+def test_layernorm_backward_refuses_a_short_workspace_and_zero_fills_for_no_tokens():
+    lib = _lib.load()
+    x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case([5, 9], 512, 7, torch.float32, torch.float32, seed=2))
+    _, stats = npa.ln_dwconv_fwd(x, cu, gam, bet, w, None)
+    need = lib.nplm_dwconv_ln_bwd_workspace_bytes(14, 512, 7, 0)
+    assert need >= 14 * 512 * 4
+    outs = [torch.empty_like(x)] + [torch.full((512, 7), 3.0, device=DEV)] + [torch.full((512,), 3.0, device=DEV) for _ in range(3)]
+    ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+    p = lambda t: None if t is None else t.data_ptr()
+    common = (p(x), p(dy), p(cu), p(stats), p(gam), p(bet), p(w), *(p(o) for o in outs))
+    assert lib.nplm_dwconv_ln_bwd(*common, p(ws), need - 256, 14, 512, 7, 2, 0, 0, 0, None) == -6      # NPLM_DWCONV_EWORKSPACE
+    assert lib.nplm_dwconv_ln_bwd(*common, p(ws), need, 14, 512, 7, 2, 0, 0, 8, None) == -9         # NPLM_DWCONV_EFLAGS
+    assert lib.nplm_dwconv_ln_bwd(*common, None, 0, 0, 512, 7, 0, 0, 0, 0, None) == 0
+    torch.cuda.synchronize()
+    for o in outs[1:]:
+        assert torch.count_nonzero(o).item() == 0
 
 
 def test_unsupported_arguments_are_refused():
