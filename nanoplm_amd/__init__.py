@@ -30,9 +30,12 @@ from .gated import (  # noqa: F401
 from .lnconv import (  # noqa: F401
     LnVarlenDWConv1dFunction,
     ln_dwconv_bwd,
+    ln_dwconv_bwd_op,
     ln_dwconv_fwd,
+    ln_dwconv_fwd_op,
     ln_supported,
     ln_varlen_dwconv,
+    ln_varlen_dwconv_compilable,
 )
 from .hygiene import conv_parameters, split_conv_parameters  # noqa: F401
 

@@ -157,6 +157,70 @@ def ln_varlen_dwconv(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, ep
     return LnVarlenDWConv1dFunction.apply(x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps, residual)
 
 
+# ---------------------------------------------------------------------------------------------
+# torch.library registration of the pair, so that a compiled model (torch.compile(dynamic=False),
+# src/nanoplm/pretraining/pure_pipeline.py:519-524) keeps one graph. Neither op synchronises the host.
+# ---------------------------------------------------------------------------------------------
+@torch.library.custom_op("nanoplm_amd::ln_dwconv_fwd", mutates_args=(), device_types="cuda")
+def ln_dwconv_fwd_op(x: torch.Tensor, cu_seqlens: torch.Tensor, ln_weight: torch.Tensor, ln_bias: Optional[torch.Tensor],
+                     weight: torch.Tensor, bias: Optional[torch.Tensor], eps: float = 1e-5,
+                     residual: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+    """(y, stats)."""
+    y, stats = ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps=eps, residual=residual)
+    return y, stats
+
+
+@ln_dwconv_fwd_op.register_fake
+def _(x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps=1e-5, residual=False):
+    return torch.empty_like(x, memory_format=torch.contiguous_format), x.new_empty((x.shape[0], 2), dtype=torch.float32)
+
+
+@torch.library.custom_op("nanoplm_amd::ln_dwconv_bwd", mutates_args=(), device_types="cuda")
+def ln_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, stats: torch.Tensor, ln_weight: torch.Tensor,
+                     ln_bias: Optional[torch.Tensor], weight: torch.Tensor,
+                     residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dln_weight, dln_bias, dw, db); dln_bias is zeros [C] without ``ln_bias`` (an op returns tensors only)."""
+    dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=residual)
+    if dbeta is None:
+        dbeta = torch.zeros_like(dg)
+    return dx, dg, dbeta, dw, db
+
+
+@ln_dwconv_bwd_op.register_fake
+def _(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=False):
+    C, K = weight.shape
+    f = lambda *shape: x.new_empty(shape, dtype=torch.float32)
+    return torch.empty_like(x, memory_format=torch.contiguous_format), f(C), f(C), f(C, K), f(C)
+
+
+def _ln_setup_context(ctx, inputs, output):
+    x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps, residual = inputs
+    ctx.save_for_backward(x, cu_seqlens, ln_weight, ln_bias, weight, output[1])
+    ctx.bias_dtype = None if bias is None else bias.dtype
+    ctx.residual = bool(residual)
+    ctx.set_materialize_grads(False)
+
+
+def _ln_backward(ctx, dy, _dstats):
+    x, cu_seqlens, ln_weight, ln_bias, weight, stats = ctx.saved_tensors
+    if dy is None:
+        dy = torch.zeros_like(x)
+    if dy.dtype != x.dtype:
+        dy = dy.to(x.dtype)
+    dx, dg, dbeta, dw, db = ln_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, stats, ln_weight, ln_bias, weight, ctx.residual)
+    return (dx, None, dg.to(ln_weight.dtype), None if ln_bias is None else dbeta.to(ln_bias.dtype), dw.to(weight.dtype),
+            None if ctx.bias_dtype is None else db.to(ctx.bias_dtype), None, None)
+
+
+ln_dwconv_fwd_op.register_autograd(_ln_backward, setup_context=_ln_setup_context)
+
+
+def ln_varlen_dwconv_compilable(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: float = 1e-5,
+                                residual: bool = False):
+    """Same result as :func:`ln_varlen_dwconv`, routed through the registered custom ops (traceable)."""
+    return ln_dwconv_fwd_op(x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps, residual)[0]
+
+
 def ln_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether the fused forward takes this call (K in {3,5,7,9}, rows of at most 2 KiB in multiples of 16 bytes,
     16-byte aligned contiguous x on a ROCm device). Informational: ``ln_dwconv_fwd`` finds out from the library."""

@@ -160,6 +160,53 @@ def test_layernorm_backward_refuses_a_short_workspace_and_zero_fills_for_no_toke
         assert torch.count_nonzero(o).item() == 0
 
 
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_layernorm_conv_compiles_into_one_graph(backend):
+    """The custom-op pair under torch.compile(dynamic=False) as the reference compiles its model
+    (pure_pipeline.py:519-524), a pre-norm sub-module in a bf16 residual stream: x + conv(norm(x)), then a Linear.
+    The compiled graph calls the same kernels as eager: every output and gradient bit-equal under aot_eager; Inductor
+    may fuse and re-round the elementwise ops around the opaque ops, so it is held to the eager result's tolerance."""
+    C, K = 1024, 7
+    x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case(LENS_MIX, C, K, torch.bfloat16, torch.bfloat16, seed=11))
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(C, C, bias=False).to(DEV).bfloat16()
+    params = [t.clone().requires_grad_(True) for t in (gam, bet, w, b)]
+
+    def block(x, cu):
+        h = npa.ln_varlen_dwconv_compilable(x, cu, params[0], params[1], params[2], params[3], residual=True)
+        return lin(h)
+
+    def run(fn):
+        for p in params + [lin.weight]:
+            p.grad = None
+        xin = x.clone().requires_grad_(True)
+        y = fn(xin, cu)
+        y.backward(dy)
+        return [y.detach(), xin.grad] + [p.grad.clone() for p in params + [lin.weight]]
+
+    eager = run(block)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(block, backend=backend, fullgraph=True, dynamic=False))
+    for name, a, c in zip(("y", "dx", "d ln_weight", "d ln_bias", "dw", "db", "d lin"), eager, compiled):
+        if backend == "aot_eager":
+            assert torch.equal(a, c), name
+        else:
+            err = float((a.float() - c.float()).abs().max() / a.float().abs().max().clamp_min(1e-30))
+            assert err <= 2.0 ** -7, (name, err)
+    # and the op pair agrees with the autograd.Function surface
+    xin = x.clone().requires_grad_(True)
+    y = lin(npa.ln_varlen_dwconv(xin, cu, *[p.detach() for p in params], residual=True))
+    assert torch.equal(y.detach(), eager[0])
+
+
+def test_layernorm_conv_ops_pass_opcheck():
+    x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case([5, 40, 3, 0, 90], 512, 5, torch.float32, torch.float32, seed=12))
+    torch.library.opcheck(npa.ln_dwconv_fwd_op, (x, cu, gam, bet, w, b, 1e-5, True), test_utils=("test_schema", "test_faketensor"))
+    _, stats = npa.ln_dwconv_fwd(x, cu, gam, bet, w, b)
+    torch.library.opcheck(npa.ln_dwconv_bwd_op, (x, dy, cu, stats, gam, None, w, False),
+                          test_utils=("test_schema", "test_faketensor"))
+
+
 def test_unsupported_arguments_are_refused():
     x, cu, gam, bet, w, b, dy = _case([5, 9], 64, 7, torch.float32, torch.float32, seed=1)
     with pytest.raises(RuntimeError):
