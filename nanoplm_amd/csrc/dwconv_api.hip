@@ -598,6 +598,52 @@ hipError_t static_scratch_for_current_device(void** out) {
 }  // namespace
 }  // namespace nplm
 
+// ---- LayerNorm-fused conv: shapes, geometry and the one-wave-per-row kernels' launchers ----------------------------
+namespace nplm {
+namespace {
+// rows of one 2 KiB column block: one forward kernel that takes the statistics from the tile it has staged
+bool ln_whole_rows(bool bf16, int C, int K, uintptr_t align_bits) {
+    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
+    return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
+}
+// wider rows (up to 8 KiB): a row-statistics kernel, then the conv forward that normalises as it reads
+bool ln_wide_rows(bool bf16, int C, int K, uintptr_t align_bits) {
+    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
+    return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 8192 && align_bits % 16 == 0;
+}
+// 16-byte chunks per lane of the one-wave-per-row kernels: rows of at most 2, 4, 8 KiB
+int ln_row_chunks(long long row_bytes) { return row_bytes <= 2048 ? 2 : row_bytes <= 4096 ? 4 : 8; }
+int ln_row_blocks(long long T) {
+    const int blocks = ceil_div(T, 4);
+    return blocks > kNumCU * 8 ? kNumCU * 8 : blocks;
+}
+// the default shape of a pass as an explicit geometry, whatever lds_shape_for() would pick for the width
+int make_default_lds_plan(bool bwd, bool bf16, long long T, int C, int K, LdsPlan* out) {
+    nplm_dwconv_tuning t{};
+    const LdsShapeSel sh = lds_default_shape(bwd, bf16, K);
+    t.vec = sh.vec; t.unroll = sh.rw; t.bt = sh.nrg; t.bw = sh.ncw; t.nwl = sh.nwl; t.nbuf = sh.nbuf;
+    return make_lds_plan(bwd, bf16, T, C, K, &t, out);
+}
+template <bool BF16>
+hipError_t launch_ln_stats(int nch, const void* x, float* stats, float eps, long long T, int C, hipStream_t s) {
+    const dim3 grid(ln_row_blocks(T)), block(256);
+    if (nch == 2) hipLaunchKernelGGL((ln_stats_kernel<BF16, 2>), grid, block, 0, s, x, stats, eps, (int)T, C);
+    else if (nch == 4) hipLaunchKernelGGL((ln_stats_kernel<BF16, 4>), grid, block, 0, s, x, stats, eps, (int)T, C);
+    else hipLaunchKernelGGL((ln_stats_kernel<BF16, 8>), grid, block, 0, s, x, stats, eps, (int)T, C);
+    return hipGetLastError();
+}
+template <bool BF16>
+hipError_t launch_ln_bwd_dx(int nch, const void* x, const float* stats, const void* gamma, int w_flags, const float* dn,
+                            const void* dy, void* dx, long long T, int C, hipStream_t s) {
+    const dim3 grid(ln_row_blocks(T)), block(256);
+    if (nch == 2) hipLaunchKernelGGL((ln_bwd_dx_kernel<BF16, 2>), grid, block, 0, s, x, stats, gamma, w_flags, dn, dy, dx, (int)T, C);
+    else if (nch == 4) hipLaunchKernelGGL((ln_bwd_dx_kernel<BF16, 4>), grid, block, 0, s, x, stats, gamma, w_flags, dn, dy, dx, (int)T, C);
+    else hipLaunchKernelGGL((ln_bwd_dx_kernel<BF16, 8>), grid, block, 0, s, x, stats, gamma, w_flags, dn, dy, dx, (int)T, C);
+    return hipGetLastError();
+}
+}  // namespace
+}  // namespace nplm
+
 using namespace nplm;
 
 extern "C" {
@@ -635,7 +681,7 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     return -NPLM_DWCONV_EUNSUPPORTED;
 }
 
-// ---- LayerNorm-fused forward (dwconv_ln_kernels.h) ---------------------------------------------------
+// ---- LayerNorm-fused conv (dwconv_ln_kernels.h and the NORM variants of the LDS-staged kernels) ----------------------
 int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, const void* ln_bias, float eps,
                        const void* w, const void* b, void* y, float* stats, int64_t T, int32_t C, int32_t K, int32_t S,
                        int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
@@ -650,9 +696,29 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     if (((uintptr_t)w | (uintptr_t)b | (uintptr_t)ln_weight | (uintptr_t)ln_bias) % WE || (uintptr_t)cu % 4 ||
         (uintptr_t)stats % 4 || ((uintptr_t)x | (uintptr_t)y) % E)
         return -NPLM_DWCONV_EALIGN;
-    const long long row_bytes = (long long)C * (long long)E;
-    if (!lds_ln_kernel_size(K) || row_bytes % 16 || row_bytes > kLnCbBytes || ((uintptr_t)x | (uintptr_t)y) % 16)
+    const uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
+    hipStream_t s = (hipStream_t)stream;
+    const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
+    if (ln_wide_rows(bf16, C, K, bits)) {
+        if (!stats) return -NPLM_DWCONV_ENULL;      // the statistics pass between the two kernels through it
+        LdsPlan lp;
+        rc = make_default_lds_plan(false, bf16, T, C, K, &lp);
+        if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
+        const int nch = ln_row_chunks((long long)C * (long long)E);
+        hipError_t e = bf16 ? launch_ln_stats<true>(nch, x, stats, eps, T, C, s) : launch_ln_stats<false>(nch, x, stats, eps, T, C, s);
+        if (e != hipSuccess) return (int)e;
+        const LnSide side{stats, ln_weight, ln_bias, nullptr};
+        const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+        const dim3 grid(lp.ncb * lp.nbt);
+        switch (K) {
+            case 3: return (int)launch_ln_fwd_wide_k3(bf16, la, side, g, grid, s);
+            case 5: return (int)launch_ln_fwd_wide_k5(bf16, la, side, g, grid, s);
+            case 7: return (int)launch_ln_fwd_wide_k7(bf16, la, side, g, grid, s);
+            case 9: return (int)launch_ln_fwd_wide_k9(bf16, la, side, g, grid, s);
+        }
         return -NPLM_DWCONV_EUNSUPPORTED;
+    }
+    if (!ln_whole_rows(bf16, C, K, bits)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp{};
     lp.sh = lds_ln_shape(bf16);
     lp.R = lp.sh.rw * lp.sh.nrg;
@@ -662,11 +728,9 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     lp.xcd_group = (lp.nbt % (kNumXCD * 8) == 0) ? 8 : 0;
     lp.rot_step = lp.nbt > 2 ? (int)((long long)lp.nbt * 618 / 1000) | 1 : 0;
     if (lp.rot_step >= lp.nbt) lp.rot_step = lp.nbt - 1;
-    const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
     const LnArgs ln{ln_weight, ln_bias, stats, eps};
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.nbt);
-    hipStream_t s = (hipStream_t)stream;
     switch (K) {
         case 3: return (int)launch_ln_fwd_k3(bf16, la, ln, g, grid, s);
         case 5: return (int)launch_ln_fwd_k5(bf16, la, ln, g, grid, s);
@@ -680,8 +744,7 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
 // dwconv_bwd_lds_kernel: dn, dw, db and the LayerNorm parameter sums), then the LayerNorm input gradient ---------------
 namespace {
 bool ln_supported(bool bf16, int C, int K, uintptr_t align_bits) {
-    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
-    return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
+    return ln_whole_rows(bf16, C, K, align_bits) || ln_wide_rows(bf16, C, K, align_bits);
 }
 // workspace: [conv slabs: nbt x (K+1) x C][LayerNorm slabs: nbt x 2 x C][dn: T x C fp32], each part 256-byte aligned
 struct LnBwdLayout {
@@ -689,11 +752,8 @@ struct LnBwdLayout {
     size_t conv_slabs, ln_slabs, dn, total;
 };
 int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
-    nplm_dwconv_tuning t{};
-    const LdsShapeSel sh = lds_default_shape(true, bf16, K);
-    t.vec = sh.vec; t.unroll = sh.rw; t.bt = sh.nrg; t.bw = sh.ncw; t.nwl = sh.nwl;
     LnBwdLayout l{};
-    int rc = make_lds_plan(true, bf16, T, C, K, &t, &l.lp);
+    int rc = make_default_lds_plan(true, bf16, T, C, K, &l.lp);
     if (rc) return rc;
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     l.conv_slabs = up((size_t)l.lp.nbt * (K + 1) * C * sizeof(float));
@@ -750,7 +810,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     // the conv's own residual flag stays off: the identity branch bypasses the LayerNorm and joins in the last kernel
     const int w_flags = kernel_w_flags(w_dtype, 0);
     const ConvPtrs la{x, dy, cu, w, nullptr, (void*)dn, part};
-    const LnBwdArgs ln{stats, ln_weight, ln_bias, part_ln};
+    const LnSide ln{stats, ln_weight, ln_bias, part_ln};
     const LdsGeo g = make_lds_geo(l.lp, T, C, S, w_flags);
     const dim3 grid(l.lp.ncb * l.lp.nbt);
     hipError_t e = hipErrorInvalidConfiguration;
@@ -767,16 +827,10 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     n_out = 2LL * C;      // the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
                        (const float*)part_ln, l.lp.nbt, C, 1, dln_weight, dln_bias);
-    int blocks = ceil_div(T, 4);
-    if (blocks > kNumCU * 8) blocks = kNumCU * 8;
     const void* res = (flags & NPLM_DWCONV_RESIDUAL) ? dy : nullptr;
-    if (bf16)
-        hipLaunchKernelGGL(ln_bwd_dx_kernel<true>, dim3(blocks), dim3(256), 0, s, x, stats, ln_weight, w_flags, (const float*)dn, res,
-                           dx, (int)T, C);
-    else
-        hipLaunchKernelGGL(ln_bwd_dx_kernel<false>, dim3(blocks), dim3(256), 0, s, x, stats, ln_weight, w_flags, (const float*)dn, res,
-                           dx, (int)T, C);
-    return (int)hipGetLastError();
+    const int nch = ln_row_chunks((long long)C * (long long)E);
+    return (int)(bf16 ? launch_ln_bwd_dx<true>(nch, x, stats, ln_weight, w_flags, dn, res, dx, T, C, s)
+                      : launch_ln_bwd_dx<false>(nch, x, stats, ln_weight, w_flags, dn, res, dx, T, C, s));
 }
 
 size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {

@@ -123,11 +123,16 @@ hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+// conv forward over layer_norm(x) with the statistics given (the NORM variant of dwconv_fwd_lds_kernel, default shape)
+hipError_t launch_ln_fwd_wide_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_wide_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_wide_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_wide_k9(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 // conv backward over layer_norm(x) (the NORM variant of dwconv_bwd_lds_kernel on the default backward shape)
-hipError_t launch_ln_bwd_k3(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
-hipError_t launch_ln_bwd_k5(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
-hipError_t launch_ln_bwd_k7(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
-hipError_t launch_ln_bwd_k9(bool bf16, const ConvPtrs& p, const LnBwdArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_k9(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 NPLM_DECLARE_LDS_K(3)
 NPLM_DECLARE_LDS_K(5)

@@ -300,6 +300,16 @@ __device__ __forceinline__ int pregated_offset(int lc) {
     }
 }
 
+// LayerNorm folded into the conv kernels (NORM variants below): the conv runs over n = layer_norm(x; gamma, beta), x is
+// the raw input and the row statistics come from `stats` (written by dwconv_ln_fwd_kernel or ln_stats_kernel,
+// dwconv_ln_kernels.h); the waves normalise x rows as they read them out of LDS.
+struct LnSide {
+    const float* stats;    // [T][2] fp32 (mean, rstd)
+    const void* gamma;     // [C], weight dtype
+    const void* beta;      // [C] or null
+    float* partial2;       // backward only: [nbt][2][C] partial sums of dgamma, dbeta
+};
+
 // =============================================================================================
 // Forward
 // =============================================================================================
@@ -309,10 +319,14 @@ __device__ __forceinline__ int pregated_offset(int lc) {
 // GATED: x is z = [u | g] of shape [T, 2C] (the SwiGLU MLP's Wi output, modeling.py:300-302) and the
 // conv runs over h = u * silu(g), formed in registers as rows are read out of LDS; a buffer then
 // holds a u tile followed by a g tile, and y is still [T, C].
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, int NBUF, bool GATED = false>
+//
+// NORM: y = conv(layer_norm(x)) (+ x: the residual flag then adds the raw centre row instead of raising the centre
+// tap), for rows wider than the whole-row kernel of dwconv_ln_kernels.h takes; see LnSide.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, int NBUF, bool GATED = false, bool NORM = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
-                      const void* __restrict__ b, void* __restrict__ y, const LdsGeo g) {
+                      const void* __restrict__ b, void* __restrict__ y, const LdsGeo g, const LnSide ln) {
+    static_assert(!NORM || (!GATED && K <= 9), "the LayerNorm variant is built for the plain short kernels");
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     using Row = RowVec<BF16, VEC>;
@@ -405,12 +419,22 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
         }
         if constexpr (PREGATE) gate_prepass<SH, BF16>(lds_raw, wv - SH::NWC, NWL, lane);
     } else {
-        load_weights<VEC, K>(w, g.w_flags, c0, wr);
+        load_weights<VEC, K>(w, NORM ? (g.w_flags & ~W_RESIDUAL) : g.w_flags, c0, wr);
         if (b) {
 #pragma unroll
             for (int v = 0; v < VEC; ++v)
                 bias[v] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(b)[c0 + v])
                                    : reinterpret_cast<const float*>(b)[c0 + v];
+        }
+    }
+    float gam[NORM ? VEC : 1], bet[NORM ? VEC : 1];
+    const bool add_raw = NORM && (g.w_flags & W_RESIDUAL);
+    if constexpr (NORM) {
+        const bool wb = (g.w_flags & W_BF16) != 0;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            gam[v] = wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.gamma)[c0 + v]) : reinterpret_cast<const float*>(ln.gamma)[c0 + v];
+            bet[v] = !ln.beta ? 0.f : wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.beta)[c0 + v]) : reinterpret_cast<const float*>(ln.beta)[c0 + v];
         }
     }
     bool interior = true;               // bounds of the wave's rows in the tile about to be computed
@@ -458,6 +482,29 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[u][v] = bias[v];
                 const char* lp = cur + (rg * RW) * SH::CB_BYTES + (PREGATE ? pregated_offset<SH, BF16, VEC>(lc0) : lc0 * E);
+                // LayerNorm: (rstd, -mean * rstd) of the wave's staged rows, wave-uniform; a staged row is normalised
+                // as it is read, after its raw values have joined the output row they are the centre of
+                float sa[NORM ? RW + K - 1 : 1], sb[NORM ? RW + K - 1 : 1];
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int j = 0; j < RW + K - 1; ++j) {
+                        int tr = tf - P + j;
+                        tr = tr < 0 ? 0 : tr < T ? tr : T - 1;
+                        const float mean = ln.stats[2 * (size_t)tr], rstd = ln.stats[2 * (size_t)tr + 1];
+                        sa[j] = rstd;
+                        sb[j] = -mean * rstd;
+                    }
+                }
+                auto normalise = [&](int j, float (&xr)[VEC]) {
+                    if constexpr (NORM) {
+                        if (add_raw && j >= P && j < P + RW) {
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) acc[j - P][v] += xr[v];
+                        }
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(__builtin_fmaf(xr[v], sa[j], sb[j]), gam[v], bet[v]);
+                    }
+                };
                 if (interior) {
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
@@ -465,6 +512,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         if constexpr (PREGATE) lds_read_row<false, VEC>(lp + j * SH::CB_BYTES, xr);
                         else if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
                         else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+                        normalise(j, xr);
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
@@ -531,6 +579,7 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
                         float xr[VEC];
                         if constexpr (GATED) lds_read_gated_row<BF16, VEC>(lp + j * SH::CB_BYTES, lp + SH::TILE_BYTES + j * SH::CB_BYTES, xr);
                         else lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, xr);
+                        normalise(j, xr);
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
                             if (j - u >= 0 && j - u < K) {
@@ -578,22 +627,16 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 //     du = dh * silu(g),   dg = dh * u * sig(g) * (1 + g * (1 - sig(g))),   dh = the conv's dx
 // are formed in registers from the staged u and g rows.
 //
-// NORM: the conv ran over n = layer_norm(x; gamma, beta) (statistics per row in `stats`, see dwconv_ln_kernels.h) and x is
-// the raw input: the wave normalises its x rows as it reads them, dx is the gradient with respect to n, and the
+// NORM: the conv ran over n = layer_norm(x; gamma, beta) (see LnSide) and x is
+// the raw input: the wave normalises its x rows as it reads them, dx is the gradient with respect to n (fp32), and the
 // block also sums the LayerNorm parameter gradients, which need that gradient in fp32 and the normalised rows:
 //     dgamma[c] += dn[t,c] * xhat[t,c],   dbeta[c] += dn[t,c],   xhat = (x - mean) * rstd.
 // They leave the block like dw/db, in a second slab of 2 x C floats per token block.
-struct LnBwdArgs {
-    const float* stats;    // [T][2] fp32 (mean, rstd)
-    const void* gamma;     // [C], weight dtype
-    const void* beta;      // [C] or null
-    float* partial2;       // [nbt][2][C]: dgamma, dbeta partial sums
-};
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false, bool NORM = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                       const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g,
-                      const LnBwdArgs ln) {
+                      const LnSide ln) {
     static_assert(!NORM || (WDX && WDW && !GATED), "the LayerNorm variant produces every gradient of the plain conv");
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;

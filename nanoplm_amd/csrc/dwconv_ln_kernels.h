@@ -429,8 +429,8 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
 // LayerNorm backward with respect to its input, given the gradient dn of the normalised tensor (fp32: what the NORM
 // variant of dwconv_bwd_lds_kernel writes as dx) and the row statistics of the forward:
 //     g = gamma * dn,   dx = rstd * (g - mean_c(g) - xhat * mean_c(g * xhat))  (+ dy: the residual connection's share)
-// The parameter gradients are summed by the conv backward, where dn is still in fp32. One wave per row (rows of at
-// most 2 KiB: two 16-byte chunks per lane), 4 rows per block, blocks stride over the rows; four streams of [T, C].
+// The parameter gradients are summed by the conv backward. One wave per row (NCH 16-byte chunks per lane: rows of at
+// most NCH KiB), 4 rows per block, blocks stride over the rows; four streams of [T, C].
 // ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float wave_allsum(float v) {
     v += dpp_row_ror<8>(v);
@@ -444,11 +444,57 @@ __device__ __forceinline__ float wave_allsum(float v) {
     return (a + b) + (c + d);
 }
 
-template <bool BF16>
+// Row statistics for rows the whole-row kernel above does not take: one wave per row, the row in registers (NCH
+// 16-byte chunks per lane: rows of at most NCH KiB), mean first and then the squared deviations from it.
+template <bool BF16, int NCH>
+__global__ void __launch_bounds__(256)
+ln_stats_kernel(const void* __restrict__ x, float* __restrict__ stats, float eps, int T, int C) {
+    constexpr int E = BF16 ? 2 : 4, CE = 16 / E;
+    using Chunk = RowVec<BF16, CE>;
+    const int lane = (int)(threadIdx.x & 63);
+    const int wv = wave_id();
+    const int rowb = C * E;
+    const float inv_c = 1.f / (float)C;
+    for (int t = (int)blockIdx.x * 4 + wv; t < T; t += (int)gridDim.x * 4) {
+        const char* row = reinterpret_cast<const char*>(x) + (size_t)t * rowb;
+        float v[NCH][CE];
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int off = (lane + 64 * i) * 16;
+            if (off < rowb) {
+                Chunk c;
+                c.load(row + off);
+                c.to_f32(v[i]);
+#pragma unroll
+                for (int e = 0; e < CE; ++e) s += v[i][e];
+            }
+        }
+        const float mean = wave_allsum(s) * inv_c;
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            if ((lane + 64 * i) * 16 < rowb) {
+#pragma unroll
+                for (int e = 0; e < CE; ++e) {
+                    const float d = v[i][e] - mean;
+                    q = __builtin_fmaf(d, d, q);
+                }
+            }
+        }
+        const float rstd = __builtin_amdgcn_rsqf(wave_allsum(q) * inv_c + eps);
+        if (lane == 0) {
+            stats[2 * (size_t)t] = mean;
+            stats[2 * (size_t)t + 1] = rstd;
+        }
+    }
+}
+
+template <bool BF16, int NCH>
 __global__ void __launch_bounds__(256)
 ln_bwd_dx_kernel(const void* __restrict__ x, const float* __restrict__ stats, const void* __restrict__ gamma, int w_flags,
                  const float* __restrict__ dn, const void* __restrict__ dy, void* __restrict__ dx, int T, int C) {
-    constexpr int E = BF16 ? 2 : 4, CE = 16 / E, NCH = 2;
+    constexpr int E = BF16 ? 2 : 4, CE = 16 / E;
     using Chunk = RowVec<BF16, CE>;
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();

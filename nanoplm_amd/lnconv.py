@@ -6,12 +6,17 @@ For a conv that takes the place of a sub-module of the reference's pre-norm enco
     x = x + self.attn(self.attn_norm(x), ...)      # attn_norm: nn.LayerNorm(hidden), modeling.py:264-266
 
 ``ln_varlen_dwconv(x, cu_seqlens, ln_weight, ln_bias, weight, bias, residual=True)`` returns
-``x + conv(layer_norm(x))`` from one read of x and one write of y: the kernel's blocks own whole rows (rows of at
-most 2 KiB: C <= 1024 in bf16, 512 in fp32; K in {3,5,7,9}), take the row statistics from the tile they have staged
-and normalise as they read. The normalised tensor is never stored; the kernel leaves (mean, rstd) per row for the
-backward, whose conv kernel normalises x again as it reads it, sums the LayerNorm parameter gradients beside dw and db
-and hands the gradient of the normalised tensor to one more pass over the rows for dx. Shapes the fused kernels are
-not built for (the library says so with its return code) compose elementwise normalisation, the plain HIP conv and
+``x + conv(layer_norm(x))``; the normalised tensor is never stored (K in {3,5,7,9}, rows in multiples of 16 bytes):
+
+* rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32): one kernel, one read of x and one write of y; its blocks
+  own whole rows, take the row statistics from the tile they have staged and normalise as they read;
+* rows of at most 8 KiB (fp32 hidden sizes up to 2048: the residual stream of the reference under ``torch.autocast``
+  is fp32): a row-statistics kernel, then the conv kernel normalising as it reads with the statistics given;
+* the forward leaves (mean, rstd) per row for the backward, whose conv kernel normalises x again as it reads it, sums
+  the LayerNorm parameter gradients beside dw and db and hands the gradient of the normalised tensor (fp32) to one
+  more pass over the rows for dx.
+
+Other shapes (the library says so with its return code) compose elementwise normalisation, the plain HIP conv and
 ATen's LayerNorm backward.
 """
 from __future__ import annotations
@@ -57,7 +62,7 @@ def ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: 
     ln_bias = None if ln_bias is None else ln_bias.to(wdt).contiguous()
     bias = None if bias is None else bias.to(wdt).contiguous()
     y = torch.empty_like(x)
-    stats = torch.empty((T, 2), dtype=torch.float32, device=x.device) if want_stats else None
+    stats = torch.empty((T, 2), dtype=torch.float32, device=x.device)    # also what the two kernels of wide rows share
     with _launch_on(x) as dev:
         rc = lib.nplm_dwconv_ln_fwd(_ptr(x), _ptr(cu_seqlens.contiguous()), _ptr(ln_weight), _ptr(ln_bias), float(eps),
                                     _ptr(weight), _ptr(bias), _ptr(y), _ptr(stats), T, C, K, S, _DTYPES[x.dtype],
@@ -74,7 +79,7 @@ def ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: 
             y = y + xf
         return y.to(x.dtype), (torch.cat([mean, rstd], dim=1) if want_stats else None)
     _lib.check(rc, "nplm_dwconv_ln_fwd")
-    return y, stats
+    return y, (stats if want_stats else None)
 
 
 def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, residual: bool = False):
@@ -222,9 +227,9 @@ def ln_varlen_dwconv_compilable(x, cu_seqlens, ln_weight, ln_bias, weight, bias=
 
 
 def ln_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the fused forward takes this call (K in {3,5,7,9}, rows of at most 2 KiB in multiples of 16 bytes,
+    """Whether the fused kernels take this call (K in {3,5,7,9}, rows of at most 8 KiB in multiples of 16 bytes,
     16-byte aligned contiguous x on a ROCm device). Informational: ``ln_dwconv_fwd`` finds out from the library."""
     if not (isinstance(x, torch.Tensor) and x.is_cuda and x.dim() == 2 and x.dtype in _DTYPES and weight.dtype in _DTYPES):
         return False
     rb = x.shape[1] * x.element_size()
-    return weight.shape[1] in (3, 5, 7, 9) and rb % 16 == 0 and rb <= 2048 and x.is_contiguous() and x.data_ptr() % 16 == 0
+    return weight.shape[1] in (3, 5, 7, 9) and rb % 16 == 0 and rb <= 8192 and x.is_contiguous() and x.data_ptr() % 16 == 0

@@ -51,9 +51,9 @@ class ConvLayer(nn.Module):
     """conv='hip': this library's module; conv='ref': the oracle's per-sequence conv1d loop in ``ref_dtype``;
     conv='shift': ``shifted_conv`` rounding to ``ref_dtype``."""
 
-    def __init__(self, hidden, inter, K, conv="hip", ref_dtype=None):
+    def __init__(self, hidden, inter, K, conv="hip", ref_dtype=None, fuse_norm=False):
         super().__init__()
-        self.conv_kind, self.ref_dtype = conv, ref_dtype
+        self.conv_kind, self.ref_dtype, self.fuse_norm = conv, ref_dtype, fuse_norm
         self.attn_norm = nn.LayerNorm(hidden, eps=1e-5, bias=False)
         self.mix_conv = npa.VarlenDWConv1d(hidden, K, residual=True)
         self.mix_out = nn.Linear(hidden, hidden, bias=False)
@@ -69,6 +69,13 @@ class ConvLayer(nn.Module):
         return O.ref_dwconv_varlen(x, cu, mod.weight, mod.bias, self.ref_dtype, residual=residual)
 
     def forward(self, x, cu_seqlens):
+        if self.fuse_norm:      # the mixer is conv(norm(x)): the norm runs inside the conv's kernels
+            if self.conv_kind == "hip":
+                h = npa.ln_varlen_dwconv_compilable(x, cu_seqlens, self.attn_norm.weight, self.attn_norm.bias, self.mix_conv.weight,
+                                                    self.mix_conv.bias, eps=self.attn_norm.eps)
+            else:
+                h = self._conv(self.mix_conv, self.attn_norm(x), cu_seqlens, False)
+            return self._mlp(x + self.mix_out(h), cu_seqlens)
         h = self.attn_norm(x)
         if not torch.compiler.is_compiling():
             self.seen["mix_conv_in"] = h.dtype
@@ -76,7 +83,9 @@ class ConvLayer(nn.Module):
             h = self.mix_conv(h, cu_seqlens)                     # h + conv(h), one pass
         else:
             h = self._conv(self.mix_conv, h, cu_seqlens, True)
-        x = x + self.mix_out(h)
+        return self._mlp(x + self.mix_out(h), cu_seqlens)
+
+    def _mlp(self, x, cu_seqlens):
         z = self.Wi(self.mlp_norm(x))
         if not torch.compiler.is_compiling():
             self.seen["mlp_conv_in"] = z.dtype
@@ -100,9 +109,9 @@ def _inputs(hidden, F_rows, seed):
     return x, dy, cu
 
 
-def _make(hidden, inter, K, seed):
+def _make(hidden, inter, K, seed, fuse_norm=False):
     torch.manual_seed(seed)
-    layer = ConvLayer(hidden, inter, K)
+    layer = ConvLayer(hidden, inter, K, fuse_norm=fuse_norm)
     with torch.no_grad():       # convs that do something: taps ~ N(0, 1/K)
         for c in (layer.mix_conv, layer.mlp_conv):
             c.weight.normal_(0, K ** -0.5)
@@ -124,7 +133,7 @@ def _run(layer, x, dy, cu, autocast):
 
 
 def _twin(layer, conv, ref_dtype=None, device=DEV, dtype=None):
-    t = ConvLayer(layer.mix_conv.channels, layer.mlp_conv.channels, layer.mix_conv.kernel_size, conv, ref_dtype)
+    t = ConvLayer(layer.mix_conv.channels, layer.mlp_conv.channels, layer.mix_conv.kernel_size, conv, ref_dtype, layer.fuse_norm)
     t.load_state_dict(layer.state_dict())
     t = t.to(device)
     return t.to(dtype) if dtype is not None else t
@@ -212,3 +221,43 @@ def test_layer_compiled_like_the_reference_compiles_its_model(hidden, inter, bac
         assert _rel(yc, y64) <= 2.0 ** -7
         for n in g64:
             assert _rel(gc[n], g64[n]) <= 2.0 ** -7, n
+
+
+@pytest.mark.parametrize("backend", ["eager", "aot_eager", "inductor"])
+@pytest.mark.parametrize("hidden,inter", SHAPES)
+def test_layer_with_the_norm_fused_into_the_conv(hidden, inter, backend):
+    """The mixer as conv(norm(x)) with the LayerNorm inside the conv's kernels (modeling.py:404-414: every sub-module
+    takes a pre-norm of the residual stream). Under autocast with fp32 parameters the stream is fp32: rows of 3 and
+    4 KiB, the statistics kernel + the normalising conv forward, and the fused backward. Against the float64
+    composition and against the unfused layer under the same autocast (torch's LayerNorm, then the HIP conv)."""
+    print(f"[case] layer fused norm {backend} hidden={hidden} inter={inter}", flush=True)
+    x, dy, cu = _inputs(hidden, 2048, 7)
+    layer = _make(hidden, inter, 7, 8, fuse_norm=True)
+    y64, g64 = _run(_twin(layer, "ref", torch.float64, "cpu", torch.float64), x.double(), dy.double(), cu, False)
+    xd, dyd, cud = x.to(DEV), dy.to(DEV), cu.to(DEV)
+    ref = _twin(layer, "shift", torch.bfloat16)
+    hip = layer.to(DEV)
+    assert npa.ln_supported(xd, hip.mix_conv.weight)
+    mod = hip
+    if backend != "eager":
+        torch._dynamo.reset()
+        mod = torch.compile(hip, backend=backend, fullgraph=True, dynamic=False)
+    try:
+        y, g = _run(mod, xd, dyd, cud, True)
+    except Exception as e:
+        if backend == "inductor" and "nanoplm_amd" not in str(e):
+            pytest.skip(f"Inductor cannot build on this box: {type(e).__name__}: {str(e)[:300]}")
+        raise
+    worst = {"y": _rel(y, y64), **{n: _rel(g[n], g64[n]) for n in g64}}
+    print("[parity] layer with fused norm vs float64, max error / max |ref|: " +
+          ", ".join(f"{k} {v:.2e}" for k, v in worst.items()), flush=True)
+    assert max(worst.values()) <= 2.0 ** -7, worst
+    yr, gr = _run(ref, xd, dyd, cud, True)
+    assert _rel(y, y64) <= _rel(yr, y64) * 2 + 1e-4
+    for n in g64:
+        assert _rel(g[n], g64[n]) <= _rel(gr[n], g64[n]) * 2 + 1e-4, n
+    if backend == "aot_eager":
+        ye, ge = _run(hip, xd, dyd, cud, True)
+        assert torch.equal(ye, y)
+        for n in g:
+            assert torch.equal(ge[n], g[n]), n

@@ -65,16 +65,41 @@ def test_fused_layernorm_forward_is_deterministic_and_takes_the_boundary_stress_
     assert torch.equal(y, y2)
 
 
+WIDE = [(torch.bfloat16, torch.bfloat16, 2048), (torch.float32, torch.float32, 1024), (torch.float32, torch.bfloat16, 768),
+        (torch.bfloat16, torch.float32, 1536), (torch.float32, torch.float32, 2048), (torch.bfloat16, torch.bfloat16, 1032)]
+
+
+@pytest.mark.parametrize("K", [3, 5, 7, 9])
+@pytest.mark.parametrize("dt,wdt,C", WIDE)
+def test_layernorm_forward_of_wide_rows(K, dt, wdt, C):
+    """Rows of more than 2 KiB (up to 8 KiB): the row-statistics kernel, then the conv forward that normalises as it
+    reads: 2, 3, 4, 6 and 8 column blocks, the last one partly filled, rows of 4 and 8 chunks per lane."""
+    print(f"[case] ln wide K={K} C={C} {dt} w {wdt}", flush=True)
+    _check_fwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C)[:6], f"ln wide K={K} C={C} {dt}")
+    _check_fwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False)[:6], f"ln wide residual K={K} C={C} {dt}",
+               residual=True)
+
+
+@pytest.mark.parametrize("K", [3, 7, 9])
+@pytest.mark.parametrize("dt,wdt,C", WIDE)
+def test_layernorm_backward_of_wide_rows(K, dt, wdt, C):
+    print(f"[case] ln bwd wide K={K} C={C} {dt} w {wdt}", flush=True)
+    _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd wide K={K} C={C} {dt}")
+    _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd wide residual K={K} C={C} {dt}",
+               residual=True)
+
+
 def test_shapes_outside_the_fused_kernel_compose_layer_norm_and_the_conv():
-    for (C, K, dt) in ((2048, 7, torch.bfloat16), (1024, 7, torch.float32), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
+    for (C, K, dt) in ((4104, 7, torch.bfloat16), (2052, 7, torch.float32), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
         print(f"[case] ln composed C={C} K={K} {dt}", flush=True)
         _check_fwd(*_case([5, 40, 3, 0, 90], C, K, dt, dt, seed=C + K)[:6], f"ln composed C={C} K={K}", residual=True, fused=False)
 
 
-@pytest.mark.parametrize("dt,C,residual", [(torch.bfloat16, 1024, True), (torch.float32, 512, False), (torch.bfloat16, 2048, True)])
+@pytest.mark.parametrize("dt,C,residual", [(torch.bfloat16, 1024, True), (torch.float32, 512, False), (torch.bfloat16, 2048, True),
+                                           (torch.float32, 1024, True), (torch.bfloat16, 4104, True)])
 def test_autograd_through_the_fused_kernels(dt, C, residual):
-    """Gradients of x, the LayerNorm parameters and the conv parameters against the float64 oracle (the last case
-    is a width the fused kernels do not take: same surface, composed ops)."""
+    """Gradients of x, the LayerNorm parameters and the conv parameters against the float64 oracle (whole-row kernels,
+    wide rows, and as the last case a width the fused kernels do not take: same surface, composed ops)."""
     x, cu, gam, bet, w, b, dy = _case(LENS_MIX, C, 7, dt, torch.float32, seed=C)
     y64, dx64, dg64, dh64, dw64, db64 = O.ref_ln_dwconv_grads(x, cu, gam, bet, w, b, dy, 1e-5, torch.float64, residual)
     xd = x.to(DEV).requires_grad_(True)
@@ -137,7 +162,7 @@ def test_fused_layernorm_backward_is_deterministic_and_takes_the_boundary_stress
 
 
 def test_backward_of_shapes_outside_the_fused_kernels_is_composed():
-    for (C, K, dt) in ((2048, 7, torch.bfloat16), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
+    for (C, K, dt) in ((4104, 7, torch.bfloat16), (1024, 15, torch.bfloat16), (1020, 7, torch.bfloat16)):
         print(f"[case] ln bwd composed C={C} K={K} {dt}", flush=True)
         _check_bwd(*_case([5, 40, 3, 0, 90], C, K, dt, dt, seed=C + K), f"ln bwd composed C={C} K={K}", residual=True, fused=False)
 
