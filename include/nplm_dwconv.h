@@ -63,7 +63,7 @@ extern "C" {
 #define NPLM_DWCONV_EWORKSPACE 6  /* workspace NULL, misaligned (256 B) or smaller than required */
 #define NPLM_DWCONV_ECU        7  /* check_cu: cu[0] != 0, cu decreasing, or cu[S] != T */
 #define NPLM_DWCONV_EFLAGS     9  /* unknown bits set in `flags` (8 is used by the internal tuning interface) */
-#define NPLM_DWCONV_EUNSUPPORTED 10 /* gated entry points: shape outside what the fused kernels are built for */
+#define NPLM_DWCONV_EUNSUPPORTED 10 /* gated and LayerNorm entry points: shape outside what the fused kernels are built for */
 #define NPLM_DWCONV_ESCRATCH   11 /* nplm_dwconv_bwd_static: the partial sums do not fit the static scratch */
 
 /* flags of the _ex entry points */
@@ -174,8 +174,8 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
 
 /*
  * LayerNorm fused into the forward, for a conv that takes the place of a sub-module of the reference's pre-norm
- * encoder layer (ModernBertEncoderLayer.forward, modeling.py:404-414: `x + attn(attn_norm(x))`, the norm being a
- * torch.nn.LayerNorm over the hidden dimension, modeling.py:264-266):
+ * encoder layer (ModernBertEncoderLayer.forward, modeling.py:404-438: `x + attn(attn_norm(x))`, the norm being a
+ * torch.nn.LayerNorm over the hidden dimension, modeling.py:408-414):
  *   n = layer_norm(x; ln_weight, ln_bias, eps) over the C channels of a row (statistics and n in fp32, never stored)
  *   y = conv(n; w, b)            (+ x with NPLM_DWCONV_RESIDUAL: the identity is the raw x, not n)
  *   stats (optional, may be NULL): [T][2] fp32, (mean, rstd) of every row - what a LayerNorm backward needs
@@ -191,8 +191,8 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
 
 /*
  * Backward of nplm_dwconv_ln_fwd (same shapes, same -NPLM_DWCONV_EUNSUPPORTED rule; the reference would reach it
- * through autograd over torch.nn.LayerNorm, modeling.py:264-266, followed by the conv's backward,
- * modeling.py:1246-1339). From x, the row statistics the forward wrote and dy:
+ * through autograd over torch.nn.LayerNorm, modeling.py:408-414).
+ * From x, the row statistics the forward wrote and dy:
  *   dw, db                  the conv's parameter gradients over n = layer_norm(x) (n is recomputed, never stored)
  *   dln_weight, dln_bias    the LayerNorm's parameter gradients, fp32 [C] (dln_bias may be NULL)
  *   dx                      the LayerNorm's input gradient (+ dy with NPLM_DWCONV_RESIDUAL), act_dtype

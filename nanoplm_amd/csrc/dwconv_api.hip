@@ -923,7 +923,7 @@ const char* nplm_dwconv_strerror(int code) {
         case NPLM_DWCONV_EWORKSPACE: return "nplm_dwconv: workspace NULL, not 256-byte aligned, or too small";
         case NPLM_DWCONV_ECU: return "nplm_dwconv: cu_seqlens must start at 0, be non-decreasing and end at T";
         case NPLM_DWCONV_EFLAGS: return "nplm_dwconv: unknown bits set in flags";
-        case NPLM_DWCONV_EUNSUPPORTED: return "nplm_dwconv: shape not supported by the fused gated kernels";
+        case NPLM_DWCONV_EUNSUPPORTED: return "nplm_dwconv: shape not supported by the fused (gated, LayerNorm) kernels";
         case NPLM_DWCONV_ESCRATCH: return "nplm_dwconv: the dw/db partial sums of this shape do not fit the library's static scratch (16 MiB); use nplm_dwconv_bwd_ex with a caller-owned workspace";
         case NPLM_DWCONV_ETUNING: return "nplm_dwconv: geometry override not available in this build";
     }

@@ -23,7 +23,7 @@
 // K-1 halo rows of every 16-row tile included, 2100 instructions per SIMD and tile).
 //
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); the LayerNorm is
-// torch.nn.LayerNorm's (modeling.py:264-266: eps = 1e-5, affine).
+// torch.nn.LayerNorm's (modeling.py:408-414: eps and bias from the config, 1e-5 and none by default, modeling.py:51-52).
 #pragma once
 #include "dwconv_lds_kernels.h"
 

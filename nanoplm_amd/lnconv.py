@@ -1,9 +1,9 @@
 """LayerNorm fused into the conv's forward: ``conv(layer_norm(x))`` (``+ x``) in one pass over x.
 
 For a conv that takes the place of a sub-module of the reference's pre-norm encoder layer
-(src/nanoplm/pretraining/models/modern_bert/modeling.py:404-414)::
+(src/nanoplm/pretraining/models/modern_bert/modeling.py:404-438)::
 
-    x = x + self.attn(self.attn_norm(x), ...)      # attn_norm: nn.LayerNorm(hidden), modeling.py:264-266
+    x = x + self.attn(self.attn_norm(x), ...)      # attn_norm: nn.LayerNorm(hidden), modeling.py:408-414
 
 ``ln_varlen_dwconv(x, cu_seqlens, ln_weight, ln_bias, weight, bias, residual=True)`` returns
 ``x + conv(layer_norm(x))``; the normalised tensor is never stored (K in {3,5,7,9}, rows in multiples of 16 bytes):

@@ -91,8 +91,8 @@ def ref_gated_dwconv_grads(z, cu_seqlens, weight, bias, dy, compute_dtype=torch.
 def ref_ln_dwconv_grads(x, cu_seqlens, ln_weight, ln_bias, weight, bias, dy, eps=1e-5, compute_dtype=torch.float64,
                         residual=False):
     """(y, dx, d ln_weight, d ln_bias, dw, db) of a conv sub-module in the reference's pre-norm layer
-    (``x + attn(attn_norm(x))``, modeling.py:404-414, the norm a ``torch.nn.LayerNorm`` over the hidden dimension,
-    modeling.py:264-266): ``F.layer_norm`` over the channels, then ``ref_dwconv_varlen``, plus the raw x with
+    (``x + attn(attn_norm(x))``, modeling.py:404-438, the norm a ``torch.nn.LayerNorm`` over the hidden dimension,
+    modeling.py:408-414): ``F.layer_norm`` over the channels, then ``ref_dwconv_varlen``, plus the raw x with
     ``residual``; gradients by autograd, everything in ``compute_dtype``. With ``dy=None`` only y."""
     xr = x.detach().to(compute_dtype).requires_grad_(True)
     gr = ln_weight.detach().to(compute_dtype).requires_grad_(True)

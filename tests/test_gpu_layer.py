@@ -226,7 +226,7 @@ def test_layer_compiled_like_the_reference_compiles_its_model(hidden, inter, bac
 @pytest.mark.parametrize("backend", ["eager", "aot_eager", "inductor"])
 @pytest.mark.parametrize("hidden,inter", SHAPES)
 def test_layer_with_the_norm_fused_into_the_conv(hidden, inter, backend):
-    """The mixer as conv(norm(x)) with the LayerNorm inside the conv's kernels (modeling.py:404-414: every sub-module
+    """The mixer as conv(norm(x)) with the LayerNorm inside the conv's kernels (modeling.py:404-438: every sub-module
     takes a pre-norm of the residual stream). Under autocast with fp32 parameters the stream is fp32: rows of 3 and
     4 KiB, the statistics kernel + the normalising conv forward, and the fused backward. Against the float64
     composition and against the unfused layer under the same autocast (torch's LayerNorm, then the HIP conv)."""

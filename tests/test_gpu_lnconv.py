@@ -1,5 +1,5 @@
 """LayerNorm fused into the conv's forward and backward (a conv sub-module of the reference's pre-norm layer,
-modeling.py:404-414) against the float64 oracle, through the C ABI entry points and the autograd surface."""
+modeling.py:404-438) against the float64 oracle, through the C ABI entry points and the autograd surface."""
 import pytest
 import torch
 
