@@ -70,7 +70,8 @@ def error_stats(got, ref64, dtype=None):
 
 
 def record_parity(name, stats):
-    """Keep the parity magnitudes of a run as gpurun_out/parity_<name>.json (best effort: the figures are also printed)."""
+    """Keep the parity magnitudes of a run as parity_<name>.json in the run's output folder (best effort: the figures are
+    also printed)."""
     import json
     import os
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
