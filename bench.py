@@ -136,6 +136,43 @@ def cpu_baseline(wl, sample_tokens):
     }
 
 
+def device_loop_baseline(d, passes, reps=3):
+    """The path the reference would take for this op on the same GPU without this library: one
+    ``torch.nn.functional.conv1d(groups=C)`` per sequence over the packed rows, concatenated, gradients by autograd
+    (whatever convolution library torch dispatches to). Informational: a whole step per repetition, wall clock."""
+    import torch
+    import torch.nn.functional as F
+
+    cu = d.cu_seqlens.cpu().tolist()
+    C, K = d.weight.shape
+    x = d.x.detach().clone().requires_grad_(passes == "fwd+bwd")
+    w = d.weight.detach().clone().requires_grad_(passes == "fwd+bwd")
+    b = d.bias.detach().clone().requires_grad_(passes == "fwd+bwd")
+
+    def step():
+        x.grad = w.grad = b.grad = None
+        ys = [F.conv1d(x[s:e].t().unsqueeze(0), w.to(x.dtype).unsqueeze(1), b.to(x.dtype), padding=K // 2, groups=C)[0].t()
+              for s, e in zip(cu[:-1], cu[1:]) if e > s]
+        y = torch.cat(ys, 0)
+        if passes == "fwd+bwd":
+            y.backward(d.dy)
+
+    t0 = time.perf_counter()
+    step()                      # first pass: the convolution library picks (and may build) its kernels per length
+    torch.cuda.synchronize()
+    first_s = time.perf_counter() - t0
+    ts = []
+    for _ in range(reps):
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        ts.append(time.perf_counter() - t)
+    med = statistics.median(ts)
+    return {"ms_per_step": med * 1e3, "tokens_per_s": d.x.shape[0] / med, "first_step_s": first_s, "reps": reps,
+            "sequences": len(cu) - 1, "what": f"per-sequence torch conv1d loop + autograd on the GPU, {passes}"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -154,6 +191,9 @@ def main():
     ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
     ap.add_argument("--prewarm-ms", type=float, default=1000.0,
                     help="untimed steps run for this long before the warm-up steps")
+    ap.add_argument("--device-loop", action="store_true",
+                    help="also time the per-sequence torch conv1d loop (the reference's way to this op) on the GPU; "
+                         "its first pass can take minutes while the convolution library prepares kernels per length")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample-tokens", type=int, default=65536)
     args = ap.parse_args()
@@ -389,6 +429,8 @@ def main():
         cp_us.append(ev.elapsed_us(0, 1))
     out["plain_copy_GBps"] = 2 * T * C * d.x.element_size() / statistics.median(cp_us[2:]) / 1e3
 
+    if args.device_loop and not (args.gated or args.ln):
+        out["reference_loop_on_gpu"] = device_loop_baseline(d, wl.passes)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, args.cpu_sample_tokens)
     print(json.dumps(out))
