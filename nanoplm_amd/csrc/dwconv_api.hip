@@ -746,19 +746,33 @@ namespace {
 bool ln_supported(bool bf16, int C, int K, uintptr_t align_bits) {
     return ln_whole_rows(bf16, C, K, align_bits) || ln_wide_rows(bf16, C, K, align_bits);
 }
-// workspace: [conv slabs: nbt x (K+1) x C][LayerNorm slabs: nbt x 2 x C][dn: T x C fp32], each part 256-byte aligned
+// workspace: [conv slabs: nbt x (K+1) x C][LayerNorm slabs: nbt x 2 x C][dn: T x C fp32], each part 256-byte aligned;
+// rows of one 2 KiB column block finish dx inside the conv backward (the WHOLE variant) and need no dn
 struct LnBwdLayout {
     LdsPlan lp;
+    bool whole;
     size_t conv_slabs, ln_slabs, dn, total;
 };
 int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
     LnBwdLayout l{};
-    int rc = make_default_lds_plan(true, bf16, T, C, K, &l.lp);
-    if (rc) return rc;
+    l.whole = ln_whole_rows(bf16, C, K, 0);
+    if (l.whole) {
+        l.lp.sh = lds_ln_bwd_shape(bf16, K);
+        l.lp.R = l.lp.sh.rw * l.lp.sh.nrg;
+        l.lp.ncb = 1;
+        l.lp.ntiles = ceil_div(T, l.lp.R);
+        l.lp.nbt = l.lp.ntiles < kNumCU ? l.lp.ntiles : kNumCU;
+        l.lp.xcd_group = (l.lp.nbt % (kNumXCD * 8) == 0) ? 8 : 0;
+        l.lp.rot_step = l.lp.nbt > 2 ? (int)((long long)l.lp.nbt * 618 / 1000) | 1 : 0;
+        if (l.lp.rot_step >= l.lp.nbt) l.lp.rot_step = l.lp.nbt - 1;
+    } else {
+        int rc = make_default_lds_plan(true, bf16, T, C, K, &l.lp);
+        if (rc) return rc;
+    }
     auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
     l.conv_slabs = up((size_t)l.lp.nbt * (K + 1) * C * sizeof(float));
     l.ln_slabs = up((size_t)l.lp.nbt * 2 * C * sizeof(float));
-    l.dn = up((size_t)T * C * sizeof(float));
+    l.dn = l.whole ? 0 : up((size_t)T * C * sizeof(float));
     l.total = l.conv_slabs + l.ln_slabs + l.dn;
     *out = l;
     return 0;
@@ -807,18 +821,28 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     float* part = reinterpret_cast<float*>(ws);
     float* part_ln = reinterpret_cast<float*>(ws + l.conv_slabs);
     float* dn = reinterpret_cast<float*>(ws + l.conv_slabs + l.ln_slabs);
-    // the conv's own residual flag stays off: the identity branch bypasses the LayerNorm and joins in the last kernel
-    const int w_flags = kernel_w_flags(w_dtype, 0);
-    const ConvPtrs la{x, dy, cu, w, nullptr, (void*)dn, part};
+    // the conv's own residual flag stays off: the identity branch bypasses the LayerNorm and joins where dx is formed
+    // (the WHOLE variant takes the flag to mean exactly that)
+    const int w_flags = kernel_w_flags(w_dtype, l.whole ? flags : 0);
+    const ConvPtrs la{x, dy, cu, w, nullptr, l.whole ? dx : (void*)dn, part};
     const LnSide ln{stats, ln_weight, ln_bias, part_ln};
     const LdsGeo g = make_lds_geo(l.lp, T, C, S, w_flags);
     const dim3 grid(l.lp.ncb * l.lp.nbt);
     hipError_t e = hipErrorInvalidConfiguration;
-    switch (K) {
-        case 3: e = launch_ln_bwd_k3(bf16, la, ln, g, grid, s); break;
-        case 5: e = launch_ln_bwd_k5(bf16, la, ln, g, grid, s); break;
-        case 7: e = launch_ln_bwd_k7(bf16, la, ln, g, grid, s); break;
-        case 9: e = launch_ln_bwd_k9(bf16, la, ln, g, grid, s); break;
+    if (l.whole) {
+        switch (K) {
+            case 3: e = launch_ln_bwd_whole_k3(bf16, la, ln, g, grid, s); break;
+            case 5: e = launch_ln_bwd_whole_k5(bf16, la, ln, g, grid, s); break;
+            case 7: e = launch_ln_bwd_whole_k7(bf16, la, ln, g, grid, s); break;
+            case 9: e = launch_ln_bwd_whole_k9(bf16, la, ln, g, grid, s); break;
+        }
+    } else {
+        switch (K) {
+            case 3: e = launch_ln_bwd_k3(bf16, la, ln, g, grid, s); break;
+            case 5: e = launch_ln_bwd_k5(bf16, la, ln, g, grid, s); break;
+            case 7: e = launch_ln_bwd_k7(bf16, la, ln, g, grid, s); break;
+            case 9: e = launch_ln_bwd_k9(bf16, la, ln, g, grid, s); break;
+        }
     }
     if (e != hipSuccess) return (int)e;
     long long n_out = (long long)(K + 1) * C;
@@ -827,6 +851,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     n_out = 2LL * C;      // the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
                        (const float*)part_ln, l.lp.nbt, C, 1, dln_weight, dln_bias);
+    if (l.whole) return (int)hipGetLastError();
     const void* res = (flags & NPLM_DWCONV_RESIDUAL) ? dy : nullptr;
     const int nch = ln_row_chunks((long long)C * (long long)E);
     return (int)(bf16 ? launch_ln_bwd_dx<true>(nch, x, stats, ln_weight, w_flags, dn, res, dx, T, C, s)

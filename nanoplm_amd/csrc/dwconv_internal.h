@@ -123,6 +123,14 @@ hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+// LayerNorm-fused backward for rows of one 2 KiB column block (the WHOLE variant of dwconv_bwd_lds_kernel): 8 wave-columns
+// x 4 bytes per lane, one row group of 16 rows (14 at K = 9, where 16 rows of x plus 24 of dy would not fit twice),
+// 8 loader waves; two (dy tile, x tile) pairs = 152 KiB at K = 7, plus 1 KiB for the exchange of the row sums.
+constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 16 : 14, 1, 8, 4, 2}; }
+hipError_t launch_ln_bwd_whole_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_whole_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_whole_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_whole_k9(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 // conv forward over layer_norm(x) with the statistics given (the NORM variant of dwconv_fwd_lds_kernel, default shape)
 hipError_t launch_ln_fwd_wide_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_wide_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);

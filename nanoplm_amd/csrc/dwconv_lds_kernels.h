@@ -300,6 +300,31 @@ __device__ __forceinline__ int pregated_offset(int lc) {
     }
 }
 
+// Workgroup barrier for LDS hand-over only. __syncthreads() carries release/acquire fences at workgroup scope, for
+// which the compiler waits for every outstanding vector memory operation of the wave first: a loader wave would
+// wait for the tile it has just put in flight, a compute wave for the acknowledgement of its stores. What the
+// hand-over of a tile needs is that this wave's LDS operations have completed (lgkmcnt) and, for a loader wave, the
+// landing of the tile it hands over, which it has waited for by count. The empty asm statements keep the compiler
+// from moving memory accesses across.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// Sum of v over the 64 lanes of a wave, left in lane 63 (other lanes hold partial sums): 4 rotations inside each row
+// of 16 lanes, then the row totals hop across the rows (row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3).
+__device__ __forceinline__ float wave_sum_in_last_lane(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));   // row_ror:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false));   // row_ror:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false));   // row_ror:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xF, 0xF, false));   // row_ror:1
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));   // row_bcast:15
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));   // row_bcast:31
+    return v;
+}
+
 // LayerNorm folded into the conv kernels (NORM variants below): the conv runs over n = layer_norm(x; gamma, beta), x is
 // the raw input and the row statistics come from `stats` (written by dwconv_ln_fwd_kernel or ln_stats_kernel,
 // dwconv_ln_kernels.h); the waves normalise x rows as they read them out of LDS.
@@ -632,12 +657,14 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 // block also sums the LayerNorm parameter gradients, which need that gradient in fp32 and the normalised rows:
 //     dgamma[c] += dn[t,c] * xhat[t,c],   dbeta[c] += dn[t,c],   xhat = (x - mean) * rstd.
 // They leave the block like dw/db, in a second slab of 2 x C floats per token block.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false, bool NORM = false>
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false, bool NORM = false,
+          bool WHOLE = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, const int32_t* __restrict__ cu,
                       const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g,
                       const LnSide ln) {
     static_assert(!NORM || (WDX && WDW && !GATED), "the LayerNorm variant produces every gradient of the plain conv");
+    static_assert(!WHOLE || (NORM && NRG == 1), "whole rows: the LayerNorm variant with one row group and one column block");
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     constexpr int XT_BYTES = R * SH::CB_BYTES;
@@ -684,6 +711,14 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane, 2 * P);
             if constexpr (WDW) stage_x(buf, t0, lw, NWL);
         }
+        if constexpr (WHOLE) {
+            // (mean, rstd) of the tile's rows travel with the tile: 8 bytes per row behind the buffers, one direct load
+            // (rows past the end read as zeros)
+            if (lw == 0 && lane * 16 < R * 8) {
+                char* d = lds_raw + 2 * BUF_BYTES + RW * NCW * 8 + (buf == lds_raw ? 0 : R * 8);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rows_rsrc(ln.stats, t0, T, 8), (lds_void*)d, 16, lane * 16, 0, 0, kLoadAux);
+            }
+        }
     };
 
     float wr[VEC][K];
@@ -710,8 +745,9 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         stage_both(lds_raw, tb * R);
         wait_vmem_all();
     } else {
-        if constexpr (WDX) load_weights<VEC, K>(w, g.w_flags, c0, wr);
+        if constexpr (WDX) load_weights<VEC, K>(w, WHOLE ? (g.w_flags & ~W_RESIDUAL) : g.w_flags, c0, wr);
     }
+    float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);      // WHOLE: [RW][NCW] (sum g, sum g * xhat)
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;
@@ -726,20 +762,23 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         char* cur = lds_raw + (it & 1) * BUF_BYTES;
         if (is_loader) {
             const int rn = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
-            if (rn < T) {
-                stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, rn);
-                wait_vmem_all();
-            }
+            if (rn < T) stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, rn);
+            if constexpr (WHOLE) lds_barrier();      // the compute waves' exchange of row sums, with the loads in flight
+            if (rn < T) wait_vmem_all();
         } else {
             const int tf = t0 + rg * RW;
+            // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
+            float dnv[WHOLE ? RW : 1][VEC];
+            const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RW * NCW * 8) + (it & 1) * R;
             if (tf < T) {
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
                 const char* lpx = cur + SH::TILE_BYTES + loff;     // x : staged row u <-> global row tf + u
                 const rsrc_t ro = rows_rsrc(dx, tf, T, x_row_bytes);
-                // LayerNorm: (rstd, -mean * rstd) of the wave's x rows, wave-uniform
-                float sa[NORM ? RW : 1], sb[NORM ? RW : 1];
-                if constexpr (NORM) {
+                // LayerNorm: (rstd, -mean * rstd) of the wave's x rows, wave-uniform: scalars loaded once per tile, or
+                // (WHOLE, 16 rows per wave) read out of LDS wherever a row is normalised, where the loaders have put them
+                float sa[NORM && !WHOLE ? RW : 1], sb[NORM && !WHOLE ? RW : 1];
+                if constexpr (NORM && !WHOLE) {
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
                         const int tr = tf + u < T ? tf + u : T - 1;
@@ -748,6 +787,16 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         sb[u] = -mean * rstd;
                     }
                 }
+                auto row_stats = [&](int u, float& a, float& b) {
+                    if constexpr (WHOLE) {
+                        const float2 mr = stl[rg * RW + u];
+                        a = mr.y;
+                        b = -mr.x * mr.y;
+                    } else {
+                        a = sa[NORM ? u : 0];
+                        b = sb[NORM ? u : 0];
+                    }
+                };
                 // Gated: per element of the wave's x rows, the two factors everything else needs:
                 //   gs = silu(g) / ... = g * sig(g)              (h = u * gs, du = dh * gs)
                 //   gd = u * sig(g) * (1 + g * (1 - sig(g)))     (dg = dh * gd)
@@ -768,8 +817,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     } else {
                         lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
                         if constexpr (NORM) {
+                            float a, b;
+                            row_stats(u, a, b);
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) xv[v] = __builtin_fmaf(__builtin_fmaf(xv[v], sa[u], sb[u]), gam[v], bet[v]);
+                            for (int v = 0; v < VEC; ++v) xv[v] = __builtin_fmaf(__builtin_fmaf(xv[v], a, b), gam[v], bet[v]);
                         }
                     }
                 };
@@ -799,18 +850,41 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                 // the LayerNorm parameter gradients from the fp32 gradient of n and the normalised row
 #pragma unroll
                                 for (int u = 0; u < RW; ++u) {
-                                    if (tf + u < T) {
-                                        float xr[VEC];
+                                    float xr[VEC];
+                                    if (WHOLE || tf + u < T) {
+                                        float a, b;
+                                        row_stats(u, a, b);
                                         lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
 #pragma unroll
+                                        for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(xr[v], a, b);      // xhat
+                                    }
+                                    if (tf + u < T) {
+#pragma unroll
                                         for (int v = 0; v < VEC; ++v) {
-                                            dga[v] = __builtin_fmaf(acc[u][v], __builtin_fmaf(xr[v], sa[u], sb[u]), dga[v]);
+                                            dga[v] = __builtin_fmaf(acc[u][v], xr[v], dga[v]);
                                             dbb[v] += acc[u][v];
                                         }
                                     }
+                                    if constexpr (WHOLE) {
+                                        // this lane's share of the two row sums LayerNorm's input gradient needs:
+                                        // g = gamma * dn and g * xhat over the channels
+                                        float p1 = 0.f, p2 = 0.f;
+#pragma unroll
+                                        for (int v = 0; v < VEC; ++v) {
+                                            const float gv = gam[v] * acc[u][v];
+                                            dnv[u][v] = acc[u][v];
+                                            p1 += gv;
+                                            p2 = __builtin_fmaf(gv, xr[v], p2);
+                                        }
+                                        p1 = wave_sum_in_last_lane(active ? p1 : 0.f);     // lanes past the row's end hold copies
+                                        p2 = wave_sum_in_last_lane(active ? p2 : 0.f);
+                                        if (lane == 63) red2[u * NCW + wc] = make_float2(p1, p2);
+                                    }
                                 }
                             }
-                            if constexpr (NORM) {
+                            if constexpr (WHOLE) {
+                                // dx waits for the other wave-columns' sums: after the barrier below
+                            } else if constexpr (NORM) {
                                 // the gradient of n leaves in fp32 whatever the activations are: the row pass that
                                 // turns it into dx rounds once
                                 const int nrowb = C * 4;
@@ -935,6 +1009,52 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         }
                     }
                     emit_dx(acc);
+                }
+            }
+            if constexpr (WHOLE) {
+                lds_barrier();
+                if (tf < T) {
+                    // dx = rstd * (g - mean_c(g) - xhat * mean_c(g * xhat)) (+ dy: the residual connection's share)
+                    const float inv_c = 1.f / (float)C;
+                    const bool resid = (g.w_flags & W_RESIDUAL) != 0;
+                    const char* lpc = cur + (rg * RW + P) * SH::CB_BYTES + lc0 * E;     // dy row of output row u: staged row u + P
+                    const char* lpx = cur + SH::TILE_BYTES + (rg * RW) * SH::CB_BYTES + lc0 * E;
+                    const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
+                    // lane u sums the wave-columns' shares of row u, in the order of the columns; row u's means are then
+                    // read out of that lane
+                    float s1 = 0.f, s2 = 0.f;
+                    if (lane < RW) {
+#pragma unroll
+                        for (int c = 0; c < NCW; ++c) {
+                            const float2 r = red2[lane * NCW + c];
+                            s1 += r.x;
+                            s2 += r.y;
+                        }
+                    }
+                    s1 *= inv_c;
+                    s2 *= inv_c;
+#pragma unroll
+                    for (int u = 0; u < RW; ++u) {
+                        if (tf + u < T) {
+                            const float2 mr = stl[rg * RW + u];
+                            const float rstd = mr.y, nb = -mr.x * mr.y;
+                            const float m1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s1), u));
+                            const float m2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s2), u));
+                            float o[VEC], xr[VEC];
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) o[v] = 0.f;
+                            if (resid) lds_read_row<BF16, VEC>(lpc + u * SH::CB_BYTES, o);
+                            lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) {
+                                const float xhat = __builtin_fmaf(xr[v], rstd, nb);
+                                o[v] = __builtin_fmaf(rstd, __builtin_fmaf(gam[v], dnv[u][v], -m1) - xhat * m2, o[v]);
+                            }
+                            Row orow;
+                            orow.from_f32(o);
+                            if (active) orow.bstore(ro, out_voff, u * rowb);
+                        }
+                    }
                 }
             }
             if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);

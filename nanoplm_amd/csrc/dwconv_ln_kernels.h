@@ -64,19 +64,6 @@ __device__ __forceinline__ void lds_write16_pinned(void* p, float a, float b, fl
     *(volatile __attribute__((address_space(3))) u32x4*)p = t;
 }
 
-// Workgroup barrier for LDS hand-over only. __syncthreads() carries release/acquire fences at workgroup scope, for
-// which the compiler waits for every outstanding vector memory operation of the wave first: a loader wave would
-// wait for the tile it has just put in flight, a compute wave for the acknowledgement of its stores. What the
-// hand-over of a tile needs is that this wave's LDS operations have completed (lgkmcnt) and, for a loader wave, the
-// landing of the tile it hands over, which it has waited for by count. The empty asm statements keep the compiler
-// from moving memory accesses across.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_waitcnt(0xC07F);      // lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-
 template <bool BF16, int VEC>
 __device__ __forceinline__ void lds_read_pinned_row(const char* p, float (&f)[VEC]) {
     RowVec<BF16, VEC> r;
