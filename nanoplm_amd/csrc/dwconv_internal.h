@@ -124,9 +124,12 @@ hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 // LayerNorm-fused backward for rows of one 2 KiB column block (the WHOLE variant of dwconv_bwd_lds_kernel): 8 wave-columns
-// x 4 bytes per lane, one row group of 16 rows (14 at K = 9, where 16 rows of x plus 24 of dy would not fit twice),
-// 8 loader waves; two (dy tile, x tile) pairs = 152 KiB at K = 7, plus 1 KiB for the exchange of the row sums.
-constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 16 : 14, 1, 8, 4, 2}; }
+// x 4 bytes per lane, 2 row groups of 8 rows (7 at K = 9, where 16 rows of x plus 24 of dy would not fit twice) and no
+// loader waves: all 16 waves compute, each stages its share of the next tile first. Two (dy tile, x tile) pairs =
+// 152 KiB at K = 7, plus 1.3 KiB for the exchange of the row sums and the tiles' row statistics. Measured at T=131072,
+// C=1024, K=7, bf16 (whole call): 8 compute waves of 16 rows + 4 loader waves 271 us (8 loader waves: 497 us, the
+// registers of 16 rows spill at 128 per wave; 12-row waves: 273 us).
+constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 8 : 7, 2, 8, 0, 2}; }
 hipError_t launch_ln_bwd_whole_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);

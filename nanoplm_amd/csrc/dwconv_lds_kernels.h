@@ -189,6 +189,49 @@ __device__ __forceinline__ void lds_read_row(const char* p, float (&f)[VEC]) {
     r.to_f32(f);
 }
 
+// The same through volatile address-space-3 accesses, for waves that also issue direct global->LDS loads: before an
+// ordinary LDS access the compiler waits for every outstanding vector-memory operation of the wave (it cannot tell
+// which LDS bytes a direct load writes); these accesses are left alone and the kernel orders them with its barriers.
+template <bool BF16, int VEC>
+__device__ __forceinline__ void lds_read_pinned_row(const char* p, float (&f)[VEC]) {
+    RowVec<BF16, VEC> r;
+    constexpr int NDW = RowVec<BF16, VEC>::BYTES / 4;
+    static_assert(RowVec<BF16, VEC>::BYTES % 4 == 0, "whole dwords");
+    uint32_t t[NDW];
+    if constexpr (NDW == 2) {
+        const u32x2 q = *(const volatile __attribute__((address_space(3))) u32x2*)p;
+        t[0] = q.x; t[1] = q.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < NDW; ++i) t[i] = ((const volatile __attribute__((address_space(3))) uint32_t*)p)[i];
+    }
+    __builtin_memcpy(&r, t, sizeof(t));
+    r.to_f32(f);
+}
+template <bool PIN, bool BF16, int VEC>
+__device__ __forceinline__ void lds_row(const char* p, float (&f)[VEC]) {
+    if constexpr (PIN) lds_read_pinned_row<BF16, VEC>(p, f);
+    else lds_read_row<BF16, VEC>(p, f);
+}
+template <bool PIN>
+__device__ __forceinline__ float2 lds_pair(const float2* p) {
+    if constexpr (PIN) {
+        const u32x2 q = *(const volatile __attribute__((address_space(3))) u32x2*)p;
+        return make_float2(__uint_as_float(q.x), __uint_as_float(q.y));
+    } else {
+        return *p;
+    }
+}
+template <bool PIN>
+__device__ __forceinline__ void lds_put_pair(float2* p, float a, float b) {
+    if constexpr (PIN) {
+        const u32x2 t = {__float_as_uint(a), __float_as_uint(b)};
+        *(volatile __attribute__((address_space(3))) u32x2*)p = t;
+    } else {
+        *p = make_float2(a, b);
+    }
+}
+
 // One lane's slice of a gated input row out of LDS: h[v] = u[v] * silu(g[v]).
 template <bool BF16, int VEC>
 __device__ __forceinline__ void lds_read_gated_row(const char* pu, const char* pg, float (&h)[VEC]) {
@@ -664,7 +707,12 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                       const void* __restrict__ w, void* __restrict__ dx, float* __restrict__ partial, const LdsGeo g,
                       const LnSide ln) {
     static_assert(!NORM || (WDX && WDW && !GATED), "the LayerNorm variant produces every gradient of the plain conv");
-    static_assert(!WHOLE || (NORM && NRG == 1), "whole rows: the LayerNorm variant with one row group and one column block");
+    static_assert(!WHOLE || NORM, "whole rows: the LayerNorm variant with one column block");
+    // NWL = 0: no loader waves; every wave stages its share of the next tile before it computes the current one, and
+    // all its LDS accesses are pinned (see lds_read_pinned_row)
+    constexpr bool SELF = NWL == 0;
+    constexpr int NLW = SELF ? NCW * NRG : NWL;           // waves that stage
+    static_assert(!SELF || WHOLE, "only the whole-row LayerNorm variant runs without loader waves");
     using SH = LdsShape<BF16, K, VEC, RW, NRG, NCW, NWL>;
     constexpr int P = SH::P, E = SH::E, R = SH::R;
     constexpr int XT_BYTES = R * SH::CB_BYTES;
@@ -675,7 +723,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
-    const bool is_loader = wv >= SH::NWC;
+    const bool is_loader = !SELF && wv >= SH::NWC;
     int cb, tb;
     lds_block_coords(g, cb, tb);
     const int T = g.T, S = g.S, C = g.C;
@@ -693,7 +741,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     const int lc0 = (lcol < cw) ? lcol : cw - VEC;
     const int c0 = cb * SH::CB_CH + lc0;
     const int out_voff = c0 * E;
-    const int lw = wv - SH::NWC;
+    const int lw = SELF ? wv : wv - SH::NWC;
 
     const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;    // pitch of x and dx (z and dz when gated)
     auto stage_x = [&](char* buf, int t0, int l, int nl) {
@@ -704,18 +752,18 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     };
     auto stage_both = [&](char* buf, int t0) {
         // with two or more loader waves, even ones take the dy tile and odd ones the x tile(s)
-        if constexpr (WDW && NWL >= 2) {
-            if (lw & 1) stage_x(buf, t0, lw >> 1, NWL / 2);
-            else        stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NWL + 1) / 2, lane, 2 * P);
+        if constexpr (WDW && NLW >= 2) {
+            if (lw & 1) stage_x(buf, t0, lw >> 1, NLW / 2);
+            else        stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw >> 1, (NLW + 1) / 2, lane, 2 * P);
         } else {
-            stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NWL, lane, 2 * P);
-            if constexpr (WDW) stage_x(buf, t0, lw, NWL);
+            stage_rows<SH, kLoadAuxOnceBwd>(dy, buf, t0 - P, SH::NROWS, T, row_bytes, col_byte0, valid_bytes, lw, NLW, lane, 2 * P);
+            if constexpr (WDW) stage_x(buf, t0, lw, NLW);
         }
         if constexpr (WHOLE) {
             // (mean, rstd) of the tile's rows travel with the tile: 8 bytes per row behind the buffers, one direct load
             // (rows past the end read as zeros)
             if (lw == 0 && lane * 16 < R * 8) {
-                char* d = lds_raw + 2 * BUF_BYTES + RW * NCW * 8 + (buf == lds_raw ? 0 : R * 8);
+                char* d = lds_raw + 2 * BUF_BYTES + R * NCW * 8 + (buf == lds_raw ? 0 : R * 8);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rows_rsrc(ln.stats, t0, T, 8), (lds_void*)d, 16, lane * 16, 0, 0, kLoadAux);
             }
         }
@@ -741,13 +789,12 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             bet[v] = !ln.beta ? 0.f : wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.beta)[c]) : reinterpret_cast<const float*>(ln.beta)[c];
         }
     }
-    if (is_loader) {
-        stage_both(lds_raw, tb * R);
-        wait_vmem_all();
-    } else {
+    if (SELF || is_loader) stage_both(lds_raw, tb * R);
+    if (!is_loader) {
         if constexpr (WDX) load_weights<VEC, K>(w, WHOLE ? (g.w_flags & ~W_RESIDUAL) : g.w_flags, c0, wr);
     }
-    float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);      // WHOLE: [RW][NCW] (sum g, sum g * xhat)
+    if (SELF || is_loader) wait_vmem_all();
+    float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);      // WHOLE: [R][NCW] (sum g, sum g * xhat)
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;
@@ -760,16 +807,19 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         const int t0 = lds_tile_row0(g, it, q, R);   // T when the block has no tile in the last round
         const int qn = lds_next_slot(g, q);
         char* cur = lds_raw + (it & 1) * BUF_BYTES;
-        if (is_loader) {
+        if (SELF || is_loader) {
             const int rn = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
             if (rn < T) stage_both(lds_raw + ((it + 1) & 1) * BUF_BYTES, rn);
-            if constexpr (WHOLE) lds_barrier();      // the compute waves' exchange of row sums, with the loads in flight
-            if (rn < T) wait_vmem_all();
-        } else {
+            if constexpr (!SELF) {
+                if constexpr (WHOLE) lds_barrier();      // the compute waves' exchange of row sums, with the loads in flight
+                if (rn < T) wait_vmem_all();
+            }
+        }
+        if (!is_loader) {
             const int tf = t0 + rg * RW;
             // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
             float dnv[WHOLE ? RW : 1][VEC];
-            const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RW * NCW * 8) + (it & 1) * R;
+            const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + R * NCW * 8) + (it & 1) * R;
             if (tf < T) {
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
@@ -789,7 +839,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 }
                 auto row_stats = [&](int u, float& a, float& b) {
                     if constexpr (WHOLE) {
-                        const float2 mr = stl[rg * RW + u];
+                        const float2 mr = lds_pair<SELF>(stl + rg * RW + u);
                         a = mr.y;
                         b = -mr.x * mr.y;
                     } else {
@@ -805,8 +855,8 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 auto read_x = [&](int u, float (&xv)[VEC]) {
                     if constexpr (GATED) {
                         float uu[VEC], gg[VEC];
-                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, uu);
-                        lds_read_row<BF16, VEC>(lpx + XT_BYTES + u * SH::CB_BYTES, gg);
+                        lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, uu);
+                        lds_row<SELF, BF16, VEC>(lpx + XT_BYTES + u * SH::CB_BYTES, gg);
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) {
                             const float sg = sigmoid_f32(gg[v]);
@@ -815,7 +865,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             xv[v] = uu[v] * gs[u][v];
                         }
                     } else {
-                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                        lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
                         if constexpr (NORM) {
                             float a, b;
                             row_stats(u, a, b);
@@ -854,7 +904,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                     if (WHOLE || tf + u < T) {
                                         float a, b;
                                         row_stats(u, a, b);
-                                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
+                                        lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
 #pragma unroll
                                         for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(xr[v], a, b);      // xhat
                                     }
@@ -878,7 +928,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                         }
                                         p1 = wave_sum_in_last_lane(active ? p1 : 0.f);     // lanes past the row's end hold copies
                                         p2 = wave_sum_in_last_lane(active ? p2 : 0.f);
-                                        if (lane == 63) red2[u * NCW + wc] = make_float2(p1, p2);
+                                        if (lane == 63) lds_put_pair<SELF>(red2 + (rg * RW + u) * NCW + wc, p1, p2);
                                     }
                                 }
                             }
@@ -932,7 +982,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float gr[VEC];
-                        lds_read_row<BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        lds_row<SELF, BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
                         if constexpr (WDW) {
                             if (j >= P && j < P + RW) {   // centre row of output j - P (interior: always < T)
 #pragma unroll
@@ -971,12 +1021,16 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     // one staged row ahead in registers; the scheduling fences keep the (already rare)
                     // path from hoisting every read and mask to the top and running out of registers
                     Row nxt;
-                    nxt.load(lpg);
+                    if constexpr (!SELF) nxt.load(lpg);
 #pragma unroll
                     for (int j = 0; j < RW + K - 1; ++j) {
                         float gr[VEC];
-                        nxt.to_f32(gr);
-                        if (j + 1 < RW + K - 1) nxt.load(lpg + (j + 1) * SH::CB_BYTES);
+                        if constexpr (SELF) {
+                            lds_row<true, BF16, VEC>(lpg + j * SH::CB_BYTES, gr);
+                        } else {
+                            nxt.to_f32(gr);
+                            if (j + 1 < RW + K - 1) nxt.load(lpg + (j + 1) * SH::CB_BYTES);
+                        }
                         if constexpr (WDW) {
                             if (j >= P && j < P + RW) {   // centre tap of output j - P: valid iff that row exists
                                 const bool okc = (vm[j - P] >> P) & 1u;
@@ -1013,6 +1067,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             }
             if constexpr (WHOLE) {
                 lds_barrier();
+                if constexpr (SELF) wait_vmem_all();      // this wave's share of the next tile has landed (long ago)
                 if (tf < T) {
                     // dx = rstd * (g - mean_c(g) - xhat * mean_c(g * xhat)) (+ dy: the residual connection's share)
                     const float inv_c = 1.f / (float)C;
@@ -1026,7 +1081,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     if (lane < RW) {
 #pragma unroll
                         for (int c = 0; c < NCW; ++c) {
-                            const float2 r = red2[lane * NCW + c];
+                            const float2 r = lds_pair<SELF>(red2 + (rg * RW + lane) * NCW + c);
                             s1 += r.x;
                             s2 += r.y;
                         }
@@ -1036,15 +1091,15 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
                         if (tf + u < T) {
-                            const float2 mr = stl[rg * RW + u];
+                            const float2 mr = lds_pair<SELF>(stl + rg * RW + u);
                             const float rstd = mr.y, nb = -mr.x * mr.y;
                             const float m1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s1), u));
                             const float m2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s2), u));
                             float o[VEC], xr[VEC];
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) o[v] = 0.f;
-                            if (resid) lds_read_row<BF16, VEC>(lpc + u * SH::CB_BYTES, o);
-                            lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
+                            if (resid) lds_row<SELF, BF16, VEC>(lpc + u * SH::CB_BYTES, o);
+                            lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) {
                                 const float xhat = __builtin_fmaf(xr[v], rstd, nb);
@@ -1059,7 +1114,9 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             }
             if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
         }
-        __syncthreads();
+        // SELF: every wave has waited for its share of the next tile before it stored dx, so the stores need not be
+        // acknowledged before the tile changes hands (__syncthreads() would wait for them)
+        if constexpr (SELF) lds_barrier(); else __syncthreads();
         q = qn;
     }
 

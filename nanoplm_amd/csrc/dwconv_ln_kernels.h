@@ -64,23 +64,6 @@ __device__ __forceinline__ void lds_write16_pinned(void* p, float a, float b, fl
     *(volatile __attribute__((address_space(3))) u32x4*)p = t;
 }
 
-template <bool BF16, int VEC>
-__device__ __forceinline__ void lds_read_pinned_row(const char* p, float (&f)[VEC]) {
-    RowVec<BF16, VEC> r;
-    constexpr int NDW = RowVec<BF16, VEC>::BYTES / 4;
-    static_assert(RowVec<BF16, VEC>::BYTES % 4 == 0, "whole dwords");
-    uint32_t t[NDW];
-    if constexpr (NDW == 2) {
-        const u32x2 q = *(const volatile __attribute__((address_space(3))) u32x2*)p;
-        t[0] = q.x; t[1] = q.y;
-    } else {
-#pragma unroll
-        for (int i = 0; i < NDW; ++i) t[i] = ((const volatile __attribute__((address_space(3))) uint32_t*)p)[i];
-    }
-    __builtin_memcpy(&r, t, sizeof(t));
-    r.to_f32(f);
-}
-
 template <int ROT>
 __device__ __forceinline__ float dpp_row_ror(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + ROT, 0xF, 0xF, false));
