@@ -12,9 +12,10 @@ For a conv that takes the place of a sub-module of the reference's pre-norm enco
   own whole rows, take the row statistics from the tile they have staged and normalise as they read;
 * rows of at most 8 KiB (fp32 hidden sizes up to 2048: the residual stream of the reference under ``torch.autocast``
   is fp32): a row-statistics kernel, then the conv kernel normalising as it reads with the statistics given;
-* the forward leaves (mean, rstd) per row for the backward, whose conv kernel normalises x again as it reads it, sums
-  the LayerNorm parameter gradients beside dw and db and hands the gradient of the normalised tensor (fp32) to one
-  more pass over the rows for dx.
+* the forward leaves (mean, rstd) per row for the backward, whose conv kernel normalises x again as it reads it and
+  sums the LayerNorm parameter gradients beside dw and db; for rows of at most 2 KiB its waves also exchange the row
+  sums of the LayerNorm input gradient and write dx themselves (one kernel), for wider rows it hands the gradient of
+  the normalised tensor (fp32) to one more pass over the rows.
 
 Other shapes (the library says so with its return code) compose elementwise normalisation, the plain HIP conv and
 ATen's LayerNorm backward.
@@ -87,7 +88,8 @@ def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, resid
     (dln_bias None without ``ln_bias``). ``stats`` is the forward's ``[T, 2]`` (mean, rstd).
 
     Fused shapes: the conv backward normalises x as it reads it (the normalised tensor is never stored) and sums the
-    LayerNorm parameter gradients beside dw and db; one more pass over (x, dn, dy) gives dx. Other shapes compose
+    LayerNorm parameter gradients beside dw and db; dx comes from the same kernel (rows of at most 2 KiB) or from one
+    more pass over (x, dn, dy). Other shapes compose
     elementwise normalisation in fp32, the plain HIP conv backward and ATen's LayerNorm backward."""
     T, C, K, S = _check(x, cu_seqlens, ln_weight, ln_bias, weight, None)
     if dy.shape != x.shape or dy.dtype != x.dtype or dy.device != x.device:
