@@ -785,6 +785,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             const bool wb = (g.w_flags & W_BF16) != 0;
             dga[v] = 0.f; dbb[v] = 0.f;
             const int c = c0 + v < C ? c0 + v : C - 1;
+            if (WHOLE && !active) { gam[v] = 0.f; bet[v] = 0.f; continue; }     // copies of the last channels: out of the row sums
             gam[v] = wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.gamma)[c]) : reinterpret_cast<const float*>(ln.gamma)[c];
             bet[v] = !ln.beta ? 0.f : wb ? bf16_to_f32(reinterpret_cast<const uint16_t*>(ln.beta)[c]) : reinterpret_cast<const float*>(ln.beta)[c];
         }
@@ -898,37 +899,55 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         } else {
                             if constexpr (NORM) {
                                 // the LayerNorm parameter gradients from the fp32 gradient of n and the normalised row
+                                if constexpr (WHOLE) {
+                                    // Straight-line code for all rows (no branch per row, so that the reads and the
+                                    // reductions of different rows overlap): rows past the end of the last tile get a
+                                    // zero gradient here and their statistics read as zeros, so they add nothing.
+                                    if (tf + RW > T) {
 #pragma unroll
-                                for (int u = 0; u < RW; ++u) {
-                                    float xr[VEC];
-                                    if (WHOLE || tf + u < T) {
-                                        float a, b;
-                                        row_stats(u, a, b);
-                                        lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
+                                        for (int u = 0; u < RW; ++u) {
+                                            if (tf + u >= T) {
 #pragma unroll
-                                        for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(xr[v], a, b);      // xhat
-                                    }
-                                    if (tf + u < T) {
-#pragma unroll
-                                        for (int v = 0; v < VEC; ++v) {
-                                            dga[v] = __builtin_fmaf(acc[u][v], xr[v], dga[v]);
-                                            dbb[v] += acc[u][v];
+                                                for (int v = 0; v < VEC; ++v) acc[u][v] = 0.f;
+                                            }
                                         }
                                     }
-                                    if constexpr (WHOLE) {
+#pragma unroll
+                                    for (int u = 0; u < RW; ++u) {
+                                        float xr[VEC], a, b;
+                                        row_stats(u, a, b);
+                                        lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
                                         // this lane's share of the two row sums LayerNorm's input gradient needs:
-                                        // g = gamma * dn and g * xhat over the channels
+                                        // g = gamma * dn and g * xhat over the channels (gamma is 0 in lanes past the
+                                        // row's end, which hold copies of the last channels)
                                         float p1 = 0.f, p2 = 0.f;
 #pragma unroll
                                         for (int v = 0; v < VEC; ++v) {
+                                            const float xhat = __builtin_fmaf(xr[v], a, b);
+                                            dga[v] = __builtin_fmaf(acc[u][v], xhat, dga[v]);
+                                            dbb[v] += acc[u][v];
                                             const float gv = gam[v] * acc[u][v];
                                             dnv[u][v] = acc[u][v];
                                             p1 += gv;
-                                            p2 = __builtin_fmaf(gv, xr[v], p2);
+                                            p2 = __builtin_fmaf(gv, xhat, p2);
                                         }
-                                        p1 = wave_sum_in_last_lane(active ? p1 : 0.f);     // lanes past the row's end hold copies
-                                        p2 = wave_sum_in_last_lane(active ? p2 : 0.f);
+                                        p1 = wave_sum_in_last_lane(p1);
+                                        p2 = wave_sum_in_last_lane(p2);
                                         if (lane == 63) lds_put_pair<SELF>(red2 + (rg * RW + u) * NCW + wc, p1, p2);
+                                    }
+                                } else {
+#pragma unroll
+                                    for (int u = 0; u < RW; ++u) {
+                                        if (tf + u < T) {
+                                            float xr[VEC], a, b;
+                                            row_stats(u, a, b);
+                                            lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
+#pragma unroll
+                                            for (int v = 0; v < VEC; ++v) {
+                                                dga[v] = __builtin_fmaf(acc[u][v], __builtin_fmaf(xr[v], a, b), dga[v]);
+                                                dbb[v] += acc[u][v];
+                                            }
+                                        }
                                     }
                                 }
                             }
@@ -1088,9 +1107,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     }
                     s1 *= inv_c;
                     s2 *= inv_c;
+                    // straight-line for all rows: the stores of rows past the end fall outside dx's buffer range
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
-                        if (tf + u < T) {
+                        {
                             const float2 mr = lds_pair<SELF>(stl + rg * RW + u);
                             const float rstd = mr.y, nb = -mr.x * mr.y;
                             const float m1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s1), u));
