@@ -233,6 +233,41 @@ def test_layernorm_conv_ops_pass_opcheck():
                           test_utils=("test_schema", "test_faketensor"))
 
 
+@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.float32, 1024)])
+def test_layernorm_conv_replays_correctly_from_a_hip_graph(dt, C):
+    """Forward and backward of both widths (whole-row kernels; statistics kernel + normalising conv + row pass) captured
+    once and replayed with new contents in the static buffers, with eager work and synchronisation between the
+    replays; every replay equals the eager result bit for bit."""
+    K = 7
+    x0, cu, gam, bet, w, b, dy0 = (t.to(DEV) for t in _case([100, 3, 512, 1, 408], C, K, dt, torch.float32, seed=21))
+    sx, sdy = torch.zeros_like(x0), torch.zeros_like(dy0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                      # warm-up outside capture
+        _, st = npa.ln_dwconv_fwd(sx, cu, gam, bet, w, b, residual=True)
+        npa.ln_dwconv_bwd(sx, sdy, cu, st, gam, bet, w, residual=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        gy, gst = npa.ln_dwconv_fwd(sx, cu, gam, bet, w, b, residual=True)
+        gout = npa.ln_dwconv_bwd(sx, sdy, cu, gst, gam, bet, w, residual=True)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    for it in range(4):
+        x = (torch.randn(x0.shape, device=DEV, generator=g) * 2 + 0.5).to(dt)
+        dy = torch.randn(x0.shape, device=DEV, generator=g).to(dt)
+        sx.copy_(x)
+        sdy.copy_(dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        ey, est = npa.ln_dwconv_fwd(x, cu, gam, bet, w, b, residual=True)
+        eout = npa.ln_dwconv_bwd(x, dy, cu, est, gam, bet, w, residual=True)
+        torch.cuda.synchronize()
+        assert torch.equal(gy, ey) and torch.equal(gst, est), f"replay {it}"
+        for a, e in zip(gout, eout):
+            assert torch.equal(a, e), f"replay {it}"
+
+
 def test_unsupported_arguments_are_refused():
     x, cu, gam, bet, w, b, dy = _case([5, 9], 64, 7, torch.float32, torch.float32, seed=1)
     with pytest.raises(RuntimeError):
