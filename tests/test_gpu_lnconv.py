@@ -173,7 +173,7 @@ def test_layernorm_backward_refuses_a_short_workspace_and_zero_fills_for_no_toke
     _, stats = npa.ln_dwconv_fwd(x, cu, gam, bet, w, None)
     need = lib.nplm_dwconv_ln_bwd_workspace_bytes(14, 512, 7, 0)
     assert need >= (7 + 1 + 2) * 512 * 4           # one token block's partial sums (whole rows: no dn buffer)
-    assert lib.nplm_dwconv_ln_bwd_workspace_bytes(14, 1024, 7, 0) >= 14 * 1024 * 4       # wide rows: dn in fp32 as well
+    assert lib.nplm_dwconv_ln_bwd_workspace_bytes(14, 2048, 7, 0) >= 14 * 2048 * 4       # rows of 8 KiB: dn in fp32 as well
     outs = [torch.empty_like(x)] + [torch.full((512, 7), 3.0, device=DEV)] + [torch.full((512,), 3.0, device=DEV) for _ in range(3)]
     ws = torch.empty(need, dtype=torch.uint8, device=DEV)
     p = lambda t: None if t is None else t.data_ptr()
