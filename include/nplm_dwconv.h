@@ -178,11 +178,15 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
  * torch.nn.LayerNorm over the hidden dimension, modeling.py:408-414):
  *   n = layer_norm(x; ln_weight, ln_bias, eps) over the C channels of a row (statistics and n in fp32, never stored)
  *   y = conv(n; w, b)            (+ x with NPLM_DWCONV_RESIDUAL: the identity is the raw x, not n)
- *   stats (optional, may be NULL): [T][2] fp32, (mean, rstd) of every row - what a LayerNorm backward needs
+ *   stats: [T][2] fp32, (mean, rstd) of every row - what nplm_dwconv_ln_bwd takes
  * x, y: act_dtype; ln_weight, ln_bias (may be NULL), w, b (may be NULL): w_dtype.
- * Built for K in {3,5,7,9} and rows that fit one 2 KiB column block (C * elemsize <= 2048 and a multiple of 16 bytes,
- * 16-byte aligned x / y), so that a block sees whole rows; anything else returns -NPLM_DWCONV_EUNSUPPORTED and
- * launches nothing (callers then run LayerNorm and nplm_dwconv_fwd_ex).
+ * Built for K in {3,5,7,9}, rows in multiples of 16 bytes and 16-byte aligned x / y:
+ *   rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32): one kernel whose blocks own whole rows and take the
+ *     statistics from the tile they have staged; `stats` may be NULL;
+ *   rows of at most 8 KiB: a row-statistics kernel, then the conv kernel normalising as it reads; `stats` is required
+ *     (it carries the statistics from the first kernel to the second; NULL returns -NPLM_DWCONV_ENULL).
+ * Anything else returns -NPLM_DWCONV_EUNSUPPORTED and launches nothing (callers then run LayerNorm and
+ * nplm_dwconv_fwd_ex).
  */
 int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, const void* ln_bias, float eps,
                        const void* w, const void* b, void* y, float* stats,
