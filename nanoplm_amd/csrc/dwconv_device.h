@@ -198,13 +198,32 @@ __host__ __device__ __forceinline__ int cu_at(const int32_t* __restrict__ cu, in
 #endif
 }
 
+// cu read through scalar loads (s_load_dword, counted by lgkmcnt). What the compiler makes of cu_at() above is a vector
+// load followed by v_readfirstlane whenever it cannot prove that nothing stored in the kernel aliases cu, and a wave
+// that waits for that load (vmcnt) also waits for every direct global->LDS load and every store it has in flight.
+// Kernels whose waves keep such operations in flight across their boundary lookups pass cu wrapped in this type.
+struct ScalarCu {
+    const int32_t* p;
+};
+__host__ __device__ __forceinline__ int cu_at(ScalarCu c, int i) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    int v;
+    const int32_t* a = c.p + i;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(a) : "memory");
+    return v;
+#else
+    return c.p[i];
+#endif
+}
+
 struct SeqCursor {
     int seq;  // index of the current interval; -1 / S for the pseudo-sequences at either end
     int cs;   // first row of the interval
     int ce;   // one past the last row
 
     // Position on the interval containing row t, searching cu[hint..S].
-    __host__ __device__ __forceinline__ void locate(const int32_t* __restrict__ cu, int S, int T, int t, int hint) {
+    template <typename CU>
+    __host__ __device__ __forceinline__ void locate(CU cu, int S, int T, int t, int hint) {
         int lo = hint < 0 ? 0 : hint, hi = S;
         // first i in [lo, S) with cu[i+1] > t, else S
         while (lo < hi) {
@@ -217,7 +236,8 @@ struct SeqCursor {
         if (cs > t) { ce = cs; cs = 0; seq = -1; }   // row lies before cu[0]
     }
     // Move forward until the interval contains row t (t must not decrease between calls).
-    __host__ __device__ __forceinline__ void advance(const int32_t* __restrict__ cu, int S, int T, int t) {
+    template <typename CU>
+    __host__ __device__ __forceinline__ void advance(CU cu, int S, int T, int t) {
         while (t >= ce && seq < S) {
             ++seq;
             cs = ce;

@@ -40,6 +40,7 @@
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); tensor contract:
 // modeling.py:339,421-439 and collator.py:322-325,405-458.
 #pragma once
+#include <type_traits>
 #include "dwconv_kernels.h"
 
 namespace nplm {
@@ -248,8 +249,8 @@ __device__ __forceinline__ void lds_read_gated_row(const char* pu, const char* p
 // Returns true when every tap of rows tf .. tf+RW-1 lies inside that one sequence. Otherwise `nce`
 // receives the end of the interval that follows the cursor's, so that crossing the (usually only)
 // boundary inside the wave's rows costs no scalar load in the middle of the tile's arithmetic.
-template <int RW, int P>
-__device__ __forceinline__ bool wave_locate(SeqCursor& sc, int& nce, const int32_t* __restrict__ cu, int S, int T, int tf) {
+template <int RW, int P, typename CU>
+__device__ __forceinline__ bool wave_locate(SeqCursor& sc, int& nce, CU cu, int S, int T, int tf) {
     if (tf >= T) return true;
     sc.locate(cu, S, T, tf, sc.seq < 0 ? 0 : sc.seq);
     const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
@@ -258,8 +259,8 @@ __device__ __forceinline__ bool wave_locate(SeqCursor& sc, int& nce, const int32
     return in;
 }
 // SeqCursor::advance that takes its first step from the prefetched `nce` (valid while `fresh`).
-__device__ __forceinline__ void advance_prefetched(SeqCursor& sq, int nce, bool& fresh, const int32_t* __restrict__ cu,
-                                                   int S, int T, int t) {
+template <typename CU>
+__device__ __forceinline__ void advance_prefetched(SeqCursor& sq, int nce, bool& fresh, CU cu, int S, int T, int t) {
     if (fresh && t >= sq.ce && sq.seq < S) {
         ++sq.seq;
         sq.cs = sq.ce;
@@ -281,9 +282,8 @@ __device__ __forceinline__ void pin_regs(float (&r)[N]) {
 // vm[u] is set iff tap row (tf + u) - P + m lies inside the sequence of output row tf + u. Rows past
 // the end of the tensor get an empty mask. `sc` (by value) must be positioned on row tf, `nce` is
 // what wave_locate left.
-template <int RW, int K>
-__device__ __forceinline__ void wave_tap_masks(SeqCursor sc, int nce, const int32_t* __restrict__ cu, int S, int T, int tf,
-                                               uint32_t (&vm)[RW]) {
+template <int RW, int K, typename CU>
+__device__ __forceinline__ void wave_tap_masks(SeqCursor sc, int nce, CU cu, int S, int T, int tf, uint32_t (&vm)[RW]) {
     bool fresh = true;
 #pragma unroll
     for (int u = 0; u < RW; ++u) {
@@ -796,11 +796,13 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     }
     if (SELF || is_loader) wait_vmem_all();
     float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);      // WHOLE: [R][NCW] (sum g, sum g * xhat)
+    // SELF: the boundary lookups go through scalar loads (see ScalarCu): the waves have stores and direct loads in flight
+    std::conditional_t<SELF, ScalarCu, const int32_t*> cuq{cu};
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;
     int nce = 0;
-    if (!is_loader) interior = wave_locate<RW, P>(sc, nce, cu, S, T, tb * R + rg * RW);
+    if (!is_loader) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, tb * R + rg * RW);
     __syncthreads();
 
     int q = tb;                         // the block's slot in round `it`
@@ -1024,7 +1026,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     // A sequence boundary falls inside the wave's window: same unrolled schedule, every
                     // tap selected (never multiplied by 0) by bit m of its output row's tap mask.
                     uint32_t vm[RW];
-                    wave_tap_masks<RW, K>(sc, nce, cu, S, T, tf, vm);
+                    wave_tap_masks<RW, K>(sc, nce, cuq, S, T, tf, vm);
                     float xc[WDW ? RW : 1][VEC];
                     if constexpr (WDW) {
 #pragma unroll
@@ -1132,7 +1134,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     }
                 }
             }
-            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
         }
         // SELF: every wave has waited for its share of the next tile before it stored dx, so the stores need not be
         // acknowledged before the tile changes hands (__syncthreads() would wait for them)
