@@ -284,6 +284,17 @@ class VarlenDWConv1d(nn.Module):
         from .gated import gated_varlen_dwconv
         return gated_varlen_dwconv(z, cu_seqlens, self.weight, self.bias, self.residual)
 
+    def forward_prenorm(self, x: torch.Tensor, cu_seqlens: torch.Tensor, norm: nn.LayerNorm) -> torch.Tensor:
+        """Pre-norm door: ``conv(norm(x))`` (``+ x`` with ``residual=True``: the identity is the raw x, as in the
+        reference's ``x + sub_module(norm(x))``, modeling.py:430-438) with ``norm`` — a ``torch.nn.LayerNorm`` over the
+        channels (modeling.py:408-414) — evaluated inside the conv's kernels (see nanoplm_amd.lnconv)."""
+        from .lnconv import ln_varlen_dwconv_compilable
+        if tuple(norm.normalized_shape) != (self.channels,):
+            raise ValueError(f"norm must normalise over the {self.channels} channels, got {tuple(norm.normalized_shape)}")
+        ln_weight = norm.weight if norm.weight is not None else torch.ones(self.channels, device=x.device, dtype=self.weight.dtype)
+        return ln_varlen_dwconv_compilable(x, cu_seqlens, ln_weight, norm.bias, self.weight, self.bias, eps=norm.eps,
+                                           residual=self.residual)
+
     def extra_repr(self) -> str:
         return (f"channels={self.channels}, kernel_size={self.kernel_size}, bias={self.bias is not None}, "
                 f"residual={self.residual}, flat_weight={self.flat_weight}, init={self.init}")

@@ -268,6 +268,29 @@ def test_layernorm_conv_replays_correctly_from_a_hip_graph(dt, C):
             assert torch.equal(a, e), f"replay {it}"
 
 
+def test_module_prenorm_door_matches_the_functional_form():
+    C, K = 512, 5
+    x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case(LENS_MIX, C, K, torch.float32, torch.float32, seed=31))
+    conv = npa.VarlenDWConv1d(C, K, residual=True).to(DEV)
+    norm = torch.nn.LayerNorm(C, eps=1e-5, bias=False).to(DEV)
+    with torch.no_grad():
+        conv.weight.copy_(w)
+        conv.bias.copy_(b)
+        norm.weight.copy_(gam)
+    xin = x.clone().requires_grad_(True)
+    y = conv.forward_prenorm(xin, cu, norm)
+    y.backward(dy)
+    y64, dx64, dg64, _, dw64, db64 = O.ref_ln_dwconv_grads(x.cpu(), cu.cpu(), gam.cpu(), None, w.cpu(), b.cpu(), dy.cpu(), 1e-5,
+                                                            torch.float64, True)
+    assert_act_close(y.detach(), y64, torch.float32, "prenorm door y")
+    assert_act_close(xin.grad, dx64, torch.float32, "prenorm door dx")
+    assert_red_close(norm.weight.grad, dg64, "prenorm door d ln_weight")
+    assert_red_close(conv.weight.grad, dw64, "prenorm door dw")
+    assert_red_close(conv.bias.grad, db64, "prenorm door db")
+    with pytest.raises(ValueError):
+        conv.forward_prenorm(xin, cu, torch.nn.LayerNorm(C + 8).to(DEV))
+
+
 def test_unsupported_arguments_are_refused():
     x, cu, gam, bet, w, b, dy = _case([5, 9], 64, 7, torch.float32, torch.float32, seed=1)
     with pytest.raises(RuntimeError):
