@@ -411,6 +411,11 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
     constexpr bool MAIL = lds_mail_fits((long long)NBUF * BUF_BYTES, SH::MAIL_BYTES);
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // NBUF x BUF_BYTES (+ MAIL_BYTES)
     int4* box = reinterpret_cast<int4*>(lds_raw + NBUF * BUF_BYTES);  // [2][NRG] (cs, ce, nce, seq)
+    // NORM: (mean, rstd) of a tile's staged rows travel with the tile, 8 bytes per row behind the buffers (and the
+    // mailbox): the compute waves read them where they normalise a row, as vector operands, instead of holding two
+    // scalars per staged row through the taps
+    constexpr int ST_BYTES = (SH::NROWS * 8 + 15) & ~15;
+    char* st_base = lds_raw + NBUF * BUF_BYTES + (MAIL ? SH::MAIL_BYTES : 0);
 
     const int lane = (int)(threadIdx.x & 63);
     const int wv = wave_id();
@@ -439,6 +444,21 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
         }
         stage_rows_fixed<SH, CNT, kLoadAuxOnceFwd>(x, buf, first_row, SH::NROWS, T, in_row_bytes, col_byte0, valid_bytes, wv - SH::NWC,
                                   NWL, lane, 2 * P);
+        if constexpr (NORM) {
+            // one dword per lane: lane l of a load takes float l of the tile's [NROWS][2] statistics (rows clamped like
+            // the tile's own)
+            if (wv == SH::NWC) {
+                const rsrc_t rst = make_rsrc(ln.stats, (uint32_t)T * 8u);
+                char* d = st_base + (buf == lds_raw ? 0 : ST_BYTES);
+#pragma unroll
+                for (int l0 = 0; l0 < SH::NROWS * 2; l0 += 64) {
+                    const int idx = l0 + lane;
+                    if (idx < SH::NROWS * 2)
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rst, (lds_void*)(d + l0 * 4), 4, (clamp_row(first_row + idx / 2, T) * 2 + (idx & 1)) * 4,
+                                                                 0, 0, kLoadAux);
+                }
+            }
+        }
         if constexpr (GATED)
             stage_rows_fixed<SH, CNT, kLoadAuxOnceFwd>(x, buf + SH::TILE_BYTES, first_row, SH::NROWS, T, in_row_bytes, rowb + col_byte0,
                                       valid_bytes, wv - SH::NWC, NWL, lane, 2 * P);
@@ -550,27 +570,19 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 #pragma unroll
                     for (int v = 0; v < VEC; ++v) acc[u][v] = bias[v];
                 const char* lp = cur + (rg * RW) * SH::CB_BYTES + (PREGATE ? pregated_offset<SH, BF16, VEC>(lc0) : lc0 * E);
-                // LayerNorm: (rstd, -mean * rstd) of the wave's staged rows, wave-uniform; a staged row is normalised
-                // as it is read, after its raw values have joined the output row they are the centre of
-                float sa[NORM ? RW + K - 1 : 1], sb[NORM ? RW + K - 1 : 1];
-                if constexpr (NORM) {
-#pragma unroll
-                    for (int j = 0; j < RW + K - 1; ++j) {
-                        int tr = tf - P + j;
-                        tr = tr < 0 ? 0 : tr < T ? tr : T - 1;
-                        const float mean = ln.stats[2 * (size_t)tr], rstd = ln.stats[2 * (size_t)tr + 1];
-                        sa[j] = rstd;
-                        sb[j] = -mean * rstd;
-                    }
-                }
+                // LayerNorm: a staged row is normalised as it is read, after its raw values have joined the output row they
+                // are the centre of
+                const float2* stq = reinterpret_cast<const float2*>(st_base + bcur * ST_BYTES) + rg * RW;
                 auto normalise = [&](int j, float (&xr)[VEC]) {
                     if constexpr (NORM) {
                         if (add_raw && j >= P && j < P + RW) {
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) acc[j - P][v] += xr[v];
                         }
+                        const float2 mr = stq[j];
+                        const float a = mr.y, b2 = -mr.x * mr.y;
 #pragma unroll
-                        for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(__builtin_fmaf(xr[v], sa[j], sb[j]), gam[v], bet[v]);
+                        for (int v = 0; v < VEC; ++v) xr[v] = __builtin_fmaf(__builtin_fmaf(xr[v], a, b2), gam[v], bet[v]);
                     }
                 };
                 if (interior) {
