@@ -606,10 +606,10 @@ bool ln_whole_rows(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
 }
-// backward only: fp32 rows of up to 4 KiB also fit a block (16 wave-columns), see lds_ln_bwd_wide_shape()
+// backward only: rows of up to 4 KiB also fit a block (16 wave-columns), see lds_ln_bwd_wide_shape()
 bool ln_bwd_whole_4k(bool bf16, int C, int K, uintptr_t align_bits) {
-    const long long row_bytes = (long long)C * 4;
-    return !bf16 && lds_ln_bwd_wide_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 4096 &&
+    const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
+    return lds_ln_bwd_wide_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 4096 &&
            align_bits % 16 == 0;
 }
 // wider rows (up to 8 KiB): a row-statistics kernel, then the conv forward that normalises as it reads
@@ -756,7 +756,7 @@ bool ln_supported(bool bf16, int C, int K, uintptr_t align_bits) {
 // rows of one 2 KiB column block finish dx inside the conv backward (the WHOLE variant) and need no dn
 struct LnBwdLayout {
     LdsPlan lp;
-    bool whole, whole4k;      // dx inside the conv backward: rows of one 2 KiB column block; fp32 rows of one 4 KiB block
+    bool whole, whole4k;      // dx inside the conv backward: rows of one 2 KiB column block; rows of one 4 KiB block
     size_t conv_slabs, ln_slabs, dn, total;
 };
 int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
@@ -764,7 +764,7 @@ int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
     l.whole4k = ln_bwd_whole_4k(bf16, C, K, 0);
     l.whole = l.whole4k || ln_whole_rows(bf16, C, K, 0);
     if (l.whole) {
-        l.lp.sh = l.whole4k ? lds_ln_bwd_wide_shape(K) : lds_ln_bwd_shape(bf16, K);
+        l.lp.sh = l.whole4k ? lds_ln_bwd_wide_shape(bf16, K) : lds_ln_bwd_shape(bf16, K);
         l.lp.R = l.lp.sh.rw * l.lp.sh.nrg;
         l.lp.ncb = 1;
         l.lp.ntiles = ceil_div(T, l.lp.R);
@@ -838,9 +838,9 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     hipError_t e = hipErrorInvalidConfiguration;
     if (l.whole4k) {
         switch (K) {
-            case 3: e = launch_ln_bwd_whole4k_k3(la, ln, g, grid, s); break;
-            case 5: e = launch_ln_bwd_whole4k_k5(la, ln, g, grid, s); break;
-            case 7: e = launch_ln_bwd_whole4k_k7(la, ln, g, grid, s); break;
+            case 3: e = launch_ln_bwd_whole4k_k3(bf16, la, ln, g, grid, s); break;
+            case 5: e = launch_ln_bwd_whole4k_k5(bf16, la, ln, g, grid, s); break;
+            case 7: e = launch_ln_bwd_whole4k_k7(bf16, la, ln, g, grid, s); break;
         }
     } else if (l.whole) {
         switch (K) {
