@@ -58,6 +58,9 @@ MEASURED_TRAFFIC = {
     ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619746803,      # 1.006 x
     ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272216838,    # 1.014 x
     ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410635307,   # 1.020 x
+    # --ln (profiles/bench_cfg3_layernorm_fused_sq_hbm_counters.md); the backward figure is the fused kernel's alone
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551643596,             # 1.026 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 861070215,            # 1.069 x
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
@@ -368,7 +371,8 @@ def main():
     def roof(nbytes, samples_us, kernel):
         med = statistics.median(samples_us)
         gbps = nbytes / med / 1e3
-        traffic = None if (args.gated or args.residual or args.ln) else MEASURED_TRAFFIC.get((wl.name, kernel))
+        traffic = (MEASURED_TRAFFIC.get((wl.name, kernel, "ln")) if args.ln else
+                   None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel)))
         r = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
              "traffic": traffic, "kernel": kernel, "median_us": med, "min_us": min(samples_us),
              "avg_us": statistics.fmean(samples_us), "launches": len(samples_us), "algorithmic_bytes": nbytes}
