@@ -268,6 +268,43 @@ def test_layernorm_conv_replays_correctly_from_a_hip_graph(dt, C):
             assert torch.equal(a, e), f"replay {it}"
 
 
+def test_layernorm_conv_at_the_headline_size_against_the_composed_ops():
+    """T=131072, C=1024, K=7, bf16 with configuration 3's lengths (8192 tiles, every block 32 rounds): the fused
+    forward and the one-kernel backward against the same operator composed on the GPU in fp32 (torch's LayerNorm, this
+    library's fp32 conv kernels, which the other tests hold to the oracle, ATen's LayerNorm backward): bf16 outputs
+    within one bf16 rounding of the fp32 result where it is not tiny, parameter gradients to 1e-4 of their largest
+    value; and twice the same bits."""
+    wl = make_workload(3, with_dy=True)
+    d = wl.to(DEV)
+    g = torch.Generator().manual_seed(9)
+    gam = (1 + 0.3 * torch.randn(wl.C, generator=g)).to(DEV)
+    bet = (0.2 * torch.randn(wl.C, generator=g)).to(DEV)
+    w32, b32 = d.weight.float(), d.bias.float()
+    y, st = npa.ln_dwconv_fwd(d.x, d.cu_seqlens, gam, bet, w32, b32, residual=True)
+    out = npa.ln_dwconv_bwd(d.x, d.dy, d.cu_seqlens, st, gam, bet, w32, residual=True)
+    y2, st2 = npa.ln_dwconv_fwd(d.x, d.cu_seqlens, gam, bet, w32, b32, residual=True)
+    out2 = npa.ln_dwconv_bwd(d.x, d.dy, d.cu_seqlens, st2, gam, bet, w32, residual=True)
+    assert torch.equal(y, y2) and all(torch.equal(a, b) for a, b in zip(out, out2))
+    xf = d.x.float().requires_grad_(True)
+    gp, bp = gam.clone().requires_grad_(True), bet.clone().requires_grad_(True)
+    wp, bbp = w32.clone().requires_grad_(True), b32.clone().requires_grad_(True)
+    n = torch.nn.functional.layer_norm(xf, (wl.C,), gp, bp, 1e-5)
+    yr = xf + npa.varlen_dwconv(n, d.cu_seqlens, wp, bbp)
+    yr.backward(d.dy.float())
+
+    def act_close(got, ref, what):
+        err = (got.float() - ref).abs()
+        bound = ref.abs() * 2.0 ** -8 + 2e-2 * (ref.abs() < 8)
+        bad = int((err > bound).sum())
+        assert bad == 0, f"{what}: {bad} elements beyond one bf16 rounding (max err {float(err.max()):.3e})"
+
+    act_close(y, yr.detach(), "y")
+    act_close(out[0], xf.grad, "dx")
+    for got, ref, what in ((out[1], gp.grad, "d ln_weight"), (out[2], bp.grad, "d ln_bias"), (out[3], wp.grad, "dw"), (out[4], bbp.grad, "db")):
+        rel = float((got - ref).abs().max() / ref.abs().max())
+        assert rel <= 1e-4, (what, rel)
+
+
 def test_module_prenorm_door_matches_the_functional_form():
     C, K = 512, 5
     x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case(LENS_MIX, C, K, torch.float32, torch.float32, seed=31))
