@@ -83,6 +83,8 @@ def test_layernorm_forward_of_wide_rows(K, dt, wdt, C):
 @pytest.mark.parametrize("K", [3, 7, 9])
 @pytest.mark.parametrize("dt,wdt,C", WIDE)
 def test_layernorm_backward_of_wide_rows(K, dt, wdt, C):
+    """Rows of more than 2 KiB: the one-kernel backward with 16 wave-columns (up to 4 KiB, K <= 7) and the two-kernel
+    path (conv backward leaving the normalised tensor's gradient in fp32, then the row pass for dx)."""
     print(f"[case] ln bwd wide K={K} C={C} {dt} w {wdt}", flush=True)
     _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd wide K={K} C={C} {dt}")
     _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd wide residual K={K} C={C} {dt}",
@@ -140,9 +142,10 @@ def _check_bwd(x, cu, gam, bet, w, b, dy, what, residual=False, fused=True):
                                        (torch.float32, torch.float32, 512), (torch.float32, torch.float32, 384),
                                        (torch.bfloat16, torch.bfloat16, 8), (torch.float32, torch.bfloat16, 100)])
 def test_fused_layernorm_backward_kernel_sizes_and_widths(K, dt, wdt, C):
-    """The conv backward that normalises x as it reads, with the LayerNorm parameter sums, and the row pass for dx:
-    rows of one and two column blocks, partly filled ones, both dtypes, mixed parameter dtypes, with and without the
-    LayerNorm bias and the residual connection; lengths around the 30-row tiles and 10-row wave windows."""
+    """The one-kernel backward for rows a block owns: the conv backward normalises x as it reads, sums the LayerNorm
+    parameter gradients, exchanges the row sums between its waves and writes dx. Full and partly filled rows, one
+    16-byte chunk per row, both dtypes, mixed parameter dtypes, with and without the LayerNorm bias and the residual
+    connection; lengths around the 16-row tiles and 8-row wave windows, empty sequences."""
     print(f"[case] ln bwd K={K} C={C} {dt} w {wdt}", flush=True)
     _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd K={K} C={C} {dt}")
     _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd residual K={K} C={C} {dt}",
