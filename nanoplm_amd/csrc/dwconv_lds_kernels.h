@@ -356,16 +356,29 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("" ::: "memory");
 }
 
-// Sum of v over the 64 lanes of a wave, left in lane 63 (other lanes hold partial sums): 4 rotations inside each row
-// of 16 lanes, then the row totals hop across the rows (row_bcast:15 into rows 1 and 3, row_bcast:31 into rows 2 and 3).
-__device__ __forceinline__ float wave_sum_in_last_lane(float v) {
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false));   // row_ror:8
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false));   // row_ror:4
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false));   // row_ror:2
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xF, 0xF, false));   // row_ror:1
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));   // row_bcast:15
-    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));   // row_bcast:31
-    return v;
+// Sums of 16 values over the 64 lanes of a wave as a reduce-scatter, 40 instructions instead of 16 x 6: the two halves
+// of the wave exchange and add (v_permlane32_swap: lanes 0-31 go on with values 0-7, lanes 32-63 with 8-15), then the
+// rows of each half (v_permlane16_swap: even rows go on with the lower four of their eight values, odd rows with the
+// upper four), then four rotations inside every row of 16 lanes. Every lane of row r ends with the totals of values
+// 4r .. 4r+3.
+__device__ __forceinline__ void wave_sums16(const float (&v)[16], float (&out)[4]) {
+    typedef unsigned u2x __attribute__((ext_vector_type(2)));
+    float s1[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const u2x r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[j]), __float_as_uint(v[j + 8]), false, false);
+        s1[j] = __uint_as_float(r.x) + __uint_as_float(r.y);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u2x r = __builtin_amdgcn_permlane16_swap(__float_as_uint(s1[j]), __float_as_uint(s1[j + 4]), false, false);
+        float t = __uint_as_float(r.x) + __uint_as_float(r.y);
+        t += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(t), 0x128, 0xF, 0xF, false));   // row_ror:8
+        t += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(t), 0x124, 0xF, 0xF, false));   // row_ror:4
+        t += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(t), 0x122, 0xF, 0xF, false));   // row_ror:2
+        t += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(t), 0x121, 0xF, 0xF, false));   // row_ror:1
+        out[j] = t;
+    }
 }
 
 // LayerNorm folded into the conv kernels (NORM variants below): the conv runs over n = layer_norm(x; gamma, beta), x is
@@ -775,7 +788,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             // (mean, rstd) of the tile's rows travel with the tile: 8 bytes per row behind the buffers, one direct load
             // (rows past the end read as zeros)
             if (lw == 0 && lane * 16 < R * 8) {
-                char* d = lds_raw + 2 * BUF_BYTES + R * NCW * 8 + (buf == lds_raw ? 0 : R * 8);
+                char* d = lds_raw + 2 * BUF_BYTES + NCW * NRG * 64 + (buf == lds_raw ? 0 : R * 8);
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rows_rsrc(ln.stats, t0, T, 8), (lds_void*)d, 16, lane * 16, 0, 0, kLoadAux);
             }
         }
@@ -807,7 +820,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         if constexpr (WDX) load_weights<VEC, K>(w, WHOLE ? (g.w_flags & ~W_RESIDUAL) : g.w_flags, c0, wr);
     }
     if (SELF || is_loader) wait_vmem_all();
-    float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);      // WHOLE: [R][NCW] (sum g, sum g * xhat)
+    // WHOLE: the wave-columns' shares of the two row sums, [NCW][NRG][8 rows] x (sum g, sum g * xhat)
+    static_assert(!WHOLE || RW <= 8, "the row sums of a wave are reduced sixteen at a time");
+    constexpr int RED_BYTES = NCW * NRG * 8 * 8;
+    float2* red2 = reinterpret_cast<float2*>(lds_raw + 2 * BUF_BYTES);
     // SELF: the boundary lookups go through scalar loads (see ScalarCu): the waves have stores and direct loads in flight
     std::conditional_t<SELF, ScalarCu, const int32_t*> cuq{cu};
     SeqCursor sc;
@@ -834,7 +850,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             const int tf = t0 + rg * RW;
             // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
             float dnv[WHOLE ? RW : 1][VEC];
-            const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + R * NCW * 8) + (it & 1) * R;
+            const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RED_BYTES) + (it & 1) * R;
             if (tf < T) {
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
                 const char* lpg = cur + loff;                      // dy: staged row j <-> global row tf - P + j
@@ -926,6 +942,9 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                             }
                                         }
                                     }
+                                    float ps[16];       // (sum g, sum g * xhat) of row u at 2u, 2u + 1
+#pragma unroll
+                                    for (int i = 0; i < 16; ++i) ps[i] = 0.f;
 #pragma unroll
                                     for (int u = 0; u < RW; ++u) {
                                         float xr[VEC], a, b;
@@ -934,7 +953,6 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                         // this lane's share of the two row sums LayerNorm's input gradient needs:
                                         // g = gamma * dn and g * xhat over the channels (gamma is 0 in lanes past the
                                         // row's end, which hold copies of the last channels)
-                                        float p1 = 0.f, p2 = 0.f;
 #pragma unroll
                                         for (int v = 0; v < VEC; ++v) {
                                             const float xhat = __builtin_fmaf(xr[v], a, b);
@@ -942,12 +960,17 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                             dbb[v] += acc[u][v];
                                             const float gv = gam[v] * acc[u][v];
                                             dnv[u][v] = acc[u][v];
-                                            p1 += gv;
-                                            p2 = __builtin_fmaf(gv, xhat, p2);
+                                            ps[2 * u] += gv;
+                                            ps[2 * u + 1] = __builtin_fmaf(gv, xhat, ps[2 * u + 1]);
                                         }
-                                        p1 = wave_sum_in_last_lane(p1);
-                                        p2 = wave_sum_in_last_lane(p2);
-                                        if (lane == 63) lds_put_pair<SELF>(red2 + (rg * RW + u) * NCW + wc, p1, p2);
+                                    }
+                                    // over the wave's lanes: every lane of row r of the wave ends with the sums of rows 2r
+                                    // and 2r + 1, and the first lane of the row leaves them for the other wave-columns
+                                    float tot[4];
+                                    wave_sums16(ps, tot);
+                                    if ((lane & 15) == 0) {
+                                        const u32x4 t = {__float_as_uint(tot[0]), __float_as_uint(tot[1]), __float_as_uint(tot[2]), __float_as_uint(tot[3])};
+                                        *(volatile __attribute__((address_space(3))) u32x4*)(red2 + (wc * NRG + rg) * 8 + (lane >> 4) * 2) = t;
                                     }
                                 } else {
 #pragma unroll
@@ -1114,7 +1137,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     if (lane < RW) {
 #pragma unroll
                         for (int c = 0; c < NCW; ++c) {
-                            const float2 r = lds_pair<SELF>(red2 + (rg * RW + lane) * NCW + c);
+                            const float2 r = lds_pair<SELF>(red2 + (c * NRG + rg) * 8 + lane);
                             s1 += r.x;
                             s2 += r.y;
                         }
