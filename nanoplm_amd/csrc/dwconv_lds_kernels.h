@@ -850,6 +850,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             const int tf = t0 + rg * RW;
             // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
             float dnv[WHOLE ? RW : 1][VEC];
+            bool located = false;       // WHOLE: the next tile's boundary lookup has been done (see emit_dx)
             const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RED_BYTES) + (it & 1) * R;
             if (tf < T) {
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
@@ -907,6 +908,13 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 };
                 // write the wave's dx rows (du and dg rows of dz when gated) from the conv's input gradient
                 auto emit_dx = [&](float (&acc)[WDX ? RW : 1][VEC]) {
+                    if constexpr (WHOLE) {
+                        // The boundary lookup for the next tile (a chain of dependent scalar loads) goes here, between the
+                        // taps and the row sums, where the other waves of the SIMD are at their arithmetic and not, as at
+                        // the end of the tile, all at the same chain.
+                        if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+                        located = true;
+                    }
                     if constexpr (WDX) {
                         const int xrowb = (int)x_row_bytes;
                         if constexpr (GATED) {
@@ -1169,7 +1177,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     }
                 }
             }
-            if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+            if (!located && it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
         }
         // SELF: every wave has waited for its share of the next tile before it stored dx, so the stores need not be
         // acknowledged before the tile changes hands (__syncthreads() would wait for them)
