@@ -849,7 +849,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         if (!is_loader) {
             const int tf = t0 + rg * RW;
             // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
-            float dnv[WHOLE ? RW : 1][VEC];
+            float dnv[WHOLE ? RW : 1][VEC], xh[WHOLE ? RW : 1][VEC];       // ... and their normalised x
             bool located = false;       // WHOLE: the next tile's boundary lookup has been done (see emit_dx)
             const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RED_BYTES) + (it & 1) * R;
             if (tf < T) {
@@ -968,6 +968,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                             dbb[v] += acc[u][v];
                                             const float gv = gam[v] * acc[u][v];
                                             dnv[u][v] = acc[u][v];
+                                            xh[u][v] = xhat;
                                             ps[2 * u] += gv;
                                             ps[2 * u + 1] = __builtin_fmaf(gv, xhat, ps[2 * u + 1]);
                                         }
@@ -1137,11 +1138,10 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     const float inv_c = 1.f / (float)C;
                     const bool resid = (g.w_flags & W_RESIDUAL) != 0;
                     const char* lpc = cur + (rg * RW + P) * SH::CB_BYTES + lc0 * E;     // dy row of output row u: staged row u + P
-                    const char* lpx = cur + SH::TILE_BYTES + (rg * RW) * SH::CB_BYTES + lc0 * E;
                     const rsrc_t ro = rows_rsrc(dx, tf, T, row_bytes);
-                    // lane u sums the wave-columns' shares of row u, in the order of the columns; row u's means are then
-                    // read out of that lane
-                    float s1 = 0.f, s2 = 0.f;
+                    // lane u sums the wave-columns' shares of row u, in the order of the columns, and takes row u's rstd;
+                    // the three per-row scalars are then read out of that lane
+                    float s1 = 0.f, s2 = 0.f, ra = 0.f;
                     if (lane < RW) {
 #pragma unroll
                         for (int c = 0; c < NCW; ++c) {
@@ -1149,27 +1149,24 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             s1 += r.x;
                             s2 += r.y;
                         }
+                        ra = lds_pair<SELF>(stl + rg * RW + lane).y;
                     }
                     s1 *= inv_c;
-                    s2 *= inv_c;
+                    s2 *= -inv_c;
                     // straight-line for all rows: the stores of rows past the end fall outside dx's buffer range
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
                         {
-                            const float2 mr = lds_pair<SELF>(stl + rg * RW + u);
-                            const float rstd = mr.y, nb = -mr.x * mr.y;
                             const float m1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s1), u));
-                            const float m2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s2), u));
-                            float o[VEC], xr[VEC];
+                            const float nm2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s2), u));
+                            const float rstd = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ra), u));
+                            float o[VEC];
 #pragma unroll
                             for (int v = 0; v < VEC; ++v) o[v] = 0.f;
                             if (resid) lds_row<SELF, BF16, VEC>(lpc + u * SH::CB_BYTES, o);
-                            lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xr);
 #pragma unroll
-                            for (int v = 0; v < VEC; ++v) {
-                                const float xhat = __builtin_fmaf(xr[v], rstd, nb);
-                                o[v] = __builtin_fmaf(rstd, __builtin_fmaf(gam[v], dnv[u][v], -m1) - xhat * m2, o[v]);
-                            }
+                            for (int v = 0; v < VEC; ++v)
+                                o[v] = __builtin_fmaf(rstd, __builtin_fmaf(nm2, xh[u][v], __builtin_fmaf(gam[v], dnv[u][v], -m1)), o[v]);
                             Row orow;
                             orow.from_f32(o);
                             if (active) orow.bstore(ro, out_voff, u * rowb);
