@@ -858,12 +858,10 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
         }
     }
     if (e != hipSuccess) return (int)e;
-    long long n_out = (long long)(K + 1) * C;
-    hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, l.lp.nbt, C, K, dw, db);
-    n_out = 2LL * C;      // the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
-    hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part_ln, l.lp.nbt, C, 1, dln_weight, dln_bias);
+    // both slab sets in one launch; the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
+    const int blocks_a = (int)(((long long)(K + 1) * C + 63) / 64), blocks_b = (int)((2LL * C + 63) / 64);
+    hipLaunchKernelGGL(dwconv_finalize2_kernel<FIN_SPLIT>, dim3((unsigned)(blocks_a + blocks_b)), dim3(64 * FIN_SPLIT), 0, s,
+                       (const float*)part, (int)K, dw, db, blocks_a, (const float*)part_ln, 1, dln_weight, dln_bias, l.lp.nbt, (int)C);
     if (l.whole) return (int)hipGetLastError();
     const void* res = (flags & NPLM_DWCONV_RESIDUAL) ? dy : nullptr;
     const int nch = ln_row_chunks((long long)C * (long long)E);

@@ -493,14 +493,14 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
 // =============================================================================================
 constexpr int FIN_SPLIT = 16;
 
+// One block of the reduction: 64 consecutive (tap, channel) outputs, SPLIT groups of slabs summed in LDS.
 template <int SPLIT>
-__global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
-                                                                     float* __restrict__ dw, float* __restrict__ db) {
-    __shared__ float red[SPLIT][64];
+__device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int block, const float* __restrict__ partial, int nbt, int C,
+                                               int K, float* __restrict__ dw, float* __restrict__ db) {
     const int lane = (int)(threadIdx.x & 63);
     const int grp = (int)(threadIdx.x >> 6);
     const long long n_out = (long long)(K + 1) * C;
-    const long long o = (long long)blockIdx.x * 64 + lane;   // o = kk*C + c
+    const long long o = (long long)block * 64 + lane;   // o = kk*C + c
     const bool on = o < n_out;
     const int per = (nbt + SPLIT - 1) / SPLIT;
     const int p0 = grp * per;
@@ -530,6 +530,24 @@ __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float
         if (kk < K) { if (dw) dw[(size_t)c * K + kk] = tot; }
         else        { if (db) db[c] = tot; }
     }
+}
+
+template <int SPLIT>
+__global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
+                                                                     float* __restrict__ dw, float* __restrict__ db) {
+    __shared__ float red[SPLIT][64];
+    finalize_block<SPLIT>(red, (int)blockIdx.x, partial, nbt, C, K, dw, db);
+}
+
+// Two slab sets of the same launch in one reduction launch (the conv's dw/db and, as a conv of K2 = 1 tap, the
+// LayerNorm's parameter gradients): the first `blocks_a` blocks take set a, the rest set b.
+template <int SPLIT>
+__global__ void __launch_bounds__(64 * SPLIT)
+dwconv_finalize2_kernel(const float* __restrict__ pa, int Ka, float* __restrict__ dwa, float* __restrict__ dba, int blocks_a,
+                        const float* __restrict__ pb, int Kb, float* __restrict__ dwb, float* __restrict__ dbb, int nbt, int C) {
+    __shared__ float red[SPLIT][64];
+    if ((int)blockIdx.x < blocks_a) finalize_block<SPLIT>(red, (int)blockIdx.x, pa, nbt, C, Ka, dwa, dba);
+    else finalize_block<SPLIT>(red, (int)blockIdx.x - blocks_a, pb, nbt, C, Kb, dwb, dbb);
 }
 
 // =============================================================================================
