@@ -308,6 +308,23 @@ def test_layernorm_conv_at_the_headline_size_against_the_composed_ops():
         assert rel <= 1e-4, (what, rel)
 
 
+def test_layernorm_conv_takes_the_static_collators_cu_seqlens():
+    """Fixed-length cu_seqlens as the static-shape collator builds it (collator.py:430-450): real sequences, pad
+    pseudo-sequences up to the flat length, trailing zero-length entries; whole-row kernels and wide rows."""
+    from nanoplm_amd.workloads import static_packed_cu
+    g = torch.Generator().manual_seed(41)
+    lens = torch.randint(20, 300, (12,), generator=g)
+    real = cu_from_lengths(lens)
+    F_rows = int(real[-1]) + 700
+    cu = static_packed_cu(real, F_rows, 256, cu_len=24)
+    assert int(cu[-1]) == F_rows and int((cu[1:] == cu[:-1]).sum()) > 0
+    lens_all = (cu[1:] - cu[:-1]).tolist()
+    for dt, C in ((torch.bfloat16, 1024), (torch.float32, 1024)):
+        x, _, gam, bet, w, b, dy = _case(lens_all, C, 7, dt, torch.float32, seed=C + 1)
+        _check_fwd(x, cu, gam, bet, w, b, f"ln static cu {dt}", residual=True)
+        _check_bwd(x, cu, gam, bet, w, b, dy, f"ln bwd static cu {dt}", residual=True)
+
+
 def test_module_prenorm_door_matches_the_functional_form():
     C, K = 512, 5
     x, cu, gam, bet, w, b, dy = (t.to(DEV) for t in _case(LENS_MIX, C, K, torch.float32, torch.float32, seed=31))
