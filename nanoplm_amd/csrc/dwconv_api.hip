@@ -841,6 +841,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
             case 3: e = launch_ln_bwd_whole4k_k3(bf16, la, ln, g, grid, s); break;
             case 5: e = launch_ln_bwd_whole4k_k5(bf16, la, ln, g, grid, s); break;
             case 7: e = launch_ln_bwd_whole4k_k7(bf16, la, ln, g, grid, s); break;
+            case 9: e = launch_ln_bwd_whole4k_k9(bf16, la, ln, g, grid, s); break;
         }
     } else if (l.whole) {
         switch (K) {

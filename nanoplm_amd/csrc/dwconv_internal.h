@@ -131,14 +131,14 @@ hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 // registers of 16 rows spill at 128 per wave; 12-row waves: 273 us).
 constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 8 : 7, 2, 8, 0, 2}; }
 // The same for rows of up to 4 KiB (fp32 hidden sizes up to 1024 - the residual stream that torch.autocast leaves - and
-// bf16 up to 2048): 16 wave-columns x 4 bytes per lane, one row group of 8 (K = 3) or 6 (K = 5, 7) rows, 144 KiB of tiles.
-// An even number of rows keeps the tiles' (mean, rstd) records 16-byte aligned; K = 9 would leave 5 rows and stays with
-// the two-kernel path.
-constexpr bool lds_ln_bwd_wide_kernel_size(int K) { return K == 3 || K == 5 || K == 7; }
-constexpr LdsShapeSel lds_ln_bwd_wide_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 3 ? 8 : 6, 1, 16, 0, 2}; }
+// bf16 up to 2048): 16 wave-columns x 4 bytes per lane, one row group of 8 (K = 3), 6 (K = 5, 7) or 5 (K = 9) rows,
+// 144 KiB of tiles.
+constexpr bool lds_ln_bwd_wide_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+constexpr LdsShapeSel lds_ln_bwd_wide_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 3 ? 8 : K <= 7 ? 6 : 5, 1, 16, 0, 2}; }
 hipError_t launch_ln_bwd_whole4k_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole4k_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole4k_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_bwd_whole4k_k9(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);

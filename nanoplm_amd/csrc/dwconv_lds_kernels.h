@@ -785,11 +785,11 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             if constexpr (WDW) stage_x(buf, t0, lw, NLW);
         }
         if constexpr (WHOLE) {
-            // (mean, rstd) of the tile's rows travel with the tile: 8 bytes per row behind the buffers, one direct load
-            // (rows past the end read as zeros)
-            if (lw == 0 && lane * 16 < R * 8) {
+            // (mean, rstd) of the tile's rows travel with the tile: 8 bytes per row behind the buffers, one direct load of
+            // one dword per lane (rows past the end read as zeros)
+            if (lw == 0 && lane < R * 2) {
                 char* d = lds_raw + 2 * BUF_BYTES + NCW * NRG * 64 + (buf == lds_raw ? 0 : R * 8);
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rows_rsrc(ln.stats, t0, T, 8), (lds_void*)d, 16, lane * 16, 0, 0, kLoadAux);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rows_rsrc(ln.stats, t0, T, 8), (lds_void*)d, 4, lane * 4, 0, 0, kLoadAux);
             }
         }
     };

@@ -83,8 +83,8 @@ def test_layernorm_forward_of_wide_rows(K, dt, wdt, C):
 @pytest.mark.parametrize("K", [3, 7, 9])
 @pytest.mark.parametrize("dt,wdt,C", WIDE)
 def test_layernorm_backward_of_wide_rows(K, dt, wdt, C):
-    """Rows of more than 2 KiB: the one-kernel backward with 16 wave-columns (up to 4 KiB, K <= 7) and the two-kernel
-    path (conv backward leaving the normalised tensor's gradient in fp32, then the row pass for dx)."""
+    """Rows of more than 2 KiB: the one-kernel backward with 16 wave-columns (up to 4 KiB) and the two-kernel path
+    (conv backward leaving the normalised tensor's gradient in fp32, then the row pass for dx)."""
     print(f"[case] ln bwd wide K={K} C={C} {dt} w {wdt}", flush=True)
     _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd wide K={K} C={C} {dt}")
     _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd wide residual K={K} C={C} {dt}",
