@@ -12,7 +12,7 @@
 // Three tile buffers: one being computed, one having its statistics taken, one in flight. A loader wave stages whole
 // rows (rows lw, lw + NWL, ... of a tile), waits by count for its own loads of the tile before the newest one, and takes
 // the statistics of exactly those rows while the compute waves are on the previous tile (a row is 2 x 64 chunks of
-// 16 bytes; a lane takes mean and squared deviations of its chunks, the wave merges them, see LaneMerge) and leaves
+// 16 bytes; the rows' sums and then their squared deviations are reduced over the wave, see ln_stats_pass) and leaves
 // (rstd, -mean * rstd, mean) per staged row in LDS, together with the sequence bounds of the tile's row groups. The
 // compute waves normalise as they read (2 FMAs per value read), write (mean, rstd) of their own rows to `stats` in
 // memory, which is what a LayerNorm backward needs, and otherwise run the forward of dwconv_lds_kernels.h: unmasked
@@ -68,52 +68,38 @@ template <int ROT>
 __device__ __forceinline__ float dpp_row_ror(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + ROT, 0xF, 0xF, false));
 }
-struct LaneMerge {
-    float w[4];    // rotation step s: nb / (na + nb) (0 when both parts are empty)
-    float q[4];    // na * nb / (na + nb)
-    float gw[3];   // merging group k + 1 into groups 0..k: the same two factors, wave-uniform
-    float gq[3];
-    float n;       // values of this lane
-};
-__device__ __forceinline__ void merge_factors(float na, float nb, float& w, float& q) {
-    const float tot = na + nb;
-    w = tot > 0.f ? nb / tot : 0.f;
-    q = tot > 0.f ? na * nb / tot : 0.f;
-}
-__device__ __forceinline__ void lane_merge_setup(LaneMerge& lm, float n_own) {
-    lm.n = n_own;
-    float n = n_own;
-    { const float nb = dpp_row_ror<8>(n); merge_factors(n, nb, lm.w[0], lm.q[0]); n += nb; }
-    { const float nb = dpp_row_ror<4>(n); merge_factors(n, nb, lm.w[1], lm.q[1]); n += nb; }
-    { const float nb = dpp_row_ror<2>(n); merge_factors(n, nb, lm.w[2], lm.q[2]); n += nb; }
-    { const float nb = dpp_row_ror<1>(n); merge_factors(n, nb, lm.w[3], lm.q[3]); n += nb; }
-    float acc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(n), 0));
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-        const float nk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(n), 16 * (k + 1)));
-        merge_factors(acc, nk, lm.gw[k], lm.gq[k]);
-        acc += nk;
-    }
-}
-__device__ __forceinline__ void merge_step(float& mean, float& m2, float mb, float qb, float w, float q) {
-    const float delta = mb - mean;
-    mean = __builtin_fmaf(delta, w, mean);
-    m2 = m2 + qb + delta * delta * q;
+// Sums of up to four values over the 64 lanes of a wave as a reduce-scatter (see wave_sums16 in dwconv_lds_kernels.h):
+// the halves of the wave exchange and add (values 0, 1 stay in lanes 0-31, values 2, 3 in lanes 32-63), then the rows of
+// each half (even rows go on with the first of their two values, odd rows with the second), then four rotations inside
+// every row of 16 lanes: every lane of row r ends with the total of value r. 10 instructions for all four.
+__device__ __forceinline__ float wave_sums4(const float (&v)[4]) {
+    typedef unsigned u2x __attribute__((ext_vector_type(2)));
+    const u2x r02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[0]), __float_as_uint(v[2]), false, false);
+    const u2x r13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(v[1]), __float_as_uint(v[3]), false, false);
+    const float a = __uint_as_float(r02.x) + __uint_as_float(r02.y);
+    const float b = __uint_as_float(r13.x) + __uint_as_float(r13.y);
+    const u2x rr = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    float t = __uint_as_float(rr.x) + __uint_as_float(rr.y);
+    t += dpp_row_ror<8>(t);
+    t += dpp_row_ror<4>(t);
+    t += dpp_row_ror<2>(t);
+    t += dpp_row_ror<1>(t);
+    return t;
 }
 
-// Loader waves: statistics of the staged rows lw, lw + nlw, ... of the tile in `buf` (at most NB of them).
-// `st[j]` = (rstd, -mean * rstd, mean, 0) of staged row j. (The loader waves store nothing to memory: their
-// s_waitcnt counts loads only.)
+// Statistics of NB staged rows of a loader wave (rows lw, lw + nlw, ...): two passes over the wave's registers - the
+// rows' sums, reduced over the wave, give the means; the squared deviations from those means, reduced the same way,
+// the variances - and (rstd, -mean * rstd, mean) per row left in LDS.
 template <typename SH, bool BF16, int NB>
-__device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int lw, int nlw, int lane, int C, float eps,
-                                              const LaneMerge& lm) {
+__device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int lw, int nlw, int lane, int C, float eps) {
+    static_assert(NB <= 4, "the rows of a loader wave are reduced four at a time");
     constexpr int CE = 16 / SH::E;                        // elements per 16-byte chunk
     constexpr int NCH = SH::CB_BYTES / 1024;              // chunks per lane and row
     const int rowb = C * SH::E;
-    const float inv_n = lm.n > 0.f ? 1.f / lm.n : 0.f;
-    float mean[NB], m2[NB];
-    // A lane's part of the NB rows: straight-line code (all reads first, four partial sums per row) so that the rows'
-    // dependency chains overlap; lanes whose chunk lies past the end of a narrow row select zeros.
+    const float inv_c = 1.f / (float)C;
+    float mean[NB], var[NB];
+    // straight-line code (all reads first, four partial sums per row) so that the rows' dependency chains overlap; lanes
+    // whose chunk lies past the end of a narrow row select zeros
     auto local = [&](auto full_c) __attribute__((always_inline)) {
         constexpr bool FULL = decltype(full_c)::value;
         float v[NB][NCH][CE];
@@ -124,6 +110,7 @@ __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int l
 #pragma unroll
             for (int i = 0; i < NCH; ++i) lds_read_chunk_pinned<BF16, CE>(buf + j * SH::CB_BYTES + (lane + 64 * i) * 16, v[r][i]);
         }
+        float s[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < NB; ++r) {
             float p[4] = {0.f, 0.f, 0.f, 0.f};
@@ -136,8 +123,12 @@ __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int l
                     p[e & 3] += v[r][i][e];
                 }
             }
-            mean[r] = ((p[0] + p[1]) + (p[2] + p[3])) * inv_n;
+            s[r] = (p[0] + p[1]) + (p[2] + p[3]);
         }
+        const float tot = wave_sums4(s);
+#pragma unroll
+        for (int r = 0; r < NB; ++r) mean[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tot), 16 * r)) * inv_c;
+        float q[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < NB; ++r) {
             float p[4] = {0.f, 0.f, 0.f, 0.f};
@@ -151,26 +142,18 @@ __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int l
                     p[e & 3] = __builtin_fmaf(t, t, p[e & 3]);
                 }
             }
-            m2[r] = (p[0] + p[1]) + (p[2] + p[3]);
+            q[r] = (p[0] + p[1]) + (p[2] + p[3]);
         }
+        const float tq = wave_sums4(q);
+#pragma unroll
+        for (int r = 0; r < NB; ++r) var[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq), 16 * r)) * inv_c;
     };
     if (rowb == SH::CB_BYTES) local(std::true_type{}); else local(std::false_type{});
-    const float inv_c = 1.f / (float)C;
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
-        merge_step(mean[r], m2[r], dpp_row_ror<8>(mean[r]), dpp_row_ror<8>(m2[r]), lm.w[0], lm.q[0]);
-        merge_step(mean[r], m2[r], dpp_row_ror<4>(mean[r]), dpp_row_ror<4>(m2[r]), lm.w[1], lm.q[1]);
-        merge_step(mean[r], m2[r], dpp_row_ror<2>(mean[r]), dpp_row_ror<2>(m2[r]), lm.w[2], lm.q[2]);
-        merge_step(mean[r], m2[r], dpp_row_ror<1>(mean[r]), dpp_row_ror<1>(m2[r]), lm.w[3], lm.q[3]);
-        float mu = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mean[r]), 0));
-        float ss = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m2[r]), 0));
-#pragma unroll
-        for (int k = 0; k < 3; ++k)
-            merge_step(mu, ss, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mean[r]), 16 * (k + 1))),
-                       __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m2[r]), 16 * (k + 1))), lm.gw[k], lm.gq[k]);
         const int j = lw + r * nlw;
-        const float rstd = __builtin_amdgcn_rsqf(ss * inv_c + eps);
-        if (lane == 0 && j < SH::NROWS) lds_write16_pinned(st + j, rstd, -mu * rstd, mu, 0.f);
+        const float rstd = __builtin_amdgcn_rsqf(var[r] + eps);
+        if (lane == 0 && j < SH::NROWS) lds_write16_pinned(st + j, rstd, -mean[r] * rstd, mean[r], 0.f);
     }
 }
 
@@ -239,7 +222,6 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
 
     float wr[VEC][K];
     float bias[VEC], gam[VEC], bet[VEC];
-    LaneMerge lm;
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     // loader waves: locate the row groups of the tile that starts at row0 and post them in mailbox set `par` (a loader
@@ -263,14 +245,9 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
         stage_whole_rows<SH, NB>(x, lds_raw, tb * R - P, T, row_bytes, valid_bytes, lw, NWL, lane);
         const int r1 = ntl > 1 ? lds_tile_row0(g, 1, lds_next_slot(g, tb), R) : T;
         if (r1 < T) stage_whole_rows<SH, NB>(x, lds_raw + BUF_BYTES, r1 - P, T, row_bytes, valid_bytes, lw, NWL, lane);
-        float n_own = 0.f;                                 // values of a row in this lane's chunks
-#pragma unroll
-        for (int i = 0; i < SH::CB_BYTES / 1024; ++i)
-            if ((lane + 64 * i) * 16 < rowb) n_own += (float)(16 / E);
-        lane_merge_setup(lm, n_own);
         post_bounds(0, tb * R);
         if (r1 < T) wait_vmem_but<CNT>(); else wait_vmem_all();       // this wave's rows of tile 0 have landed
-        ln_stats_pass<SH, BF16, NB>(lds_raw, st_all, lw, NWL, lane, C, ln.eps, lm);
+        ln_stats_pass<SH, BF16, NB>(lds_raw, st_all, lw, NWL, lane, C, ln.eps);
     } else {
         load_weights<VEC, K>(w, g.w_flags & ~W_RESIDUAL, c0, wr);      // the identity is added from the raw x below
 #pragma unroll
@@ -303,7 +280,7 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
             if (r1 < T) post_bounds((it + 1) & 1, r1);
             if (r1 < T) {
                 if (r2 < T) wait_vmem_but<CNT>(); else wait_vmem_all();
-                ln_stats_pass<SH, BF16, NB>(lds_raw + b1 * BUF_BYTES, st_all + b1 * SH::NROWS, lw, NWL, lane, C, ln.eps, lm);
+                ln_stats_pass<SH, BF16, NB>(lds_raw + b1 * BUF_BYTES, st_all + b1 * SH::NROWS, lw, NWL, lane, C, ln.eps);
             }
         } else {
             const int tf = t0 + rg * RW;
