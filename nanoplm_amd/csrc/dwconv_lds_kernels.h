@@ -725,6 +725,16 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
 // block also sums the LayerNorm parameter gradients, which need that gradient in fp32 and the normalised rows:
 //     dgamma[c] += dn[t,c] * xhat[t,c],   dbeta[c] += dn[t,c],   xhat = (x - mean) * rstd.
 // They leave the block like dw/db, in a second slab of 2 x C floats per token block.
+//
+// WHOLE (with NORM; one column block that holds whole rows, NWL = 0): the block also forms LayerNorm's input gradient,
+//     dx = rstd * (g - mean_c(g) - xhat * mean_c(g * xhat))  (+ dy with the residual flag),   g = gamma * dn,
+// and dn never leaves it. A tile takes two phases around one more barrier: after the taps every wave reduces its rows'
+// shares of sum_c g and sum_c g * xhat over its lanes (wave_sums16) and leaves them in LDS; after the barrier lane u of
+// a wave adds the wave-columns' shares of row u and the wave writes dx of its rows. LDS behind the two buffers:
+// [NCW][NRG][8] x (sum g, sum g * xhat), then two sets of (mean, rstd) per tile row, which arrive with the tile.
+// There are no loader waves (SELF): every wave issues its share of the next tile's direct loads before it starts on
+// the current tile and waits for them before it stores dx; its LDS accesses are pinned (lds_read_pinned_row), its
+// boundary lookups scalar (ScalarCu), and the tile changes hands at an LDS-only barrier with the stores in flight.
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool WDX, bool WDW, bool GATED = false, bool NORM = false,
           bool WHOLE = false>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
