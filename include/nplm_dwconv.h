@@ -181,10 +181,10 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
  *   stats: [T][2] fp32, (mean, rstd) of every row - what nplm_dwconv_ln_bwd takes
  * x, y: act_dtype; ln_weight, ln_bias (may be NULL), w, b (may be NULL): w_dtype.
  * Built for K in {3,5,7,9}, rows in multiples of 16 bytes and 16-byte aligned x / y:
- *   rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32): one kernel whose blocks own whole rows and take the
- *     statistics from the tile they have staged; `stats` may be NULL;
- *   rows of at most 8 KiB: a row-statistics kernel, then the conv kernel normalising as it reads; `stats` is required
- *     (it carries the statistics from the first kernel to the second; NULL returns -NPLM_DWCONV_ENULL).
+ *   rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32) and fp32 rows of at most 4 KiB (C <= 1024): one kernel
+ *     whose blocks own whole rows and take the statistics from the tile they have staged; `stats` may be NULL;
+ *   other rows of at most 8 KiB: a row-statistics kernel, then the conv kernel normalising as it reads; `stats` is
+ *     required (it carries the statistics from the first kernel to the second; NULL returns -NPLM_DWCONV_ENULL).
  * Anything else returns -NPLM_DWCONV_EUNSUPPORTED and launches nothing (callers then run LayerNorm and
  * nplm_dwconv_fwd_ex).
  */

@@ -606,7 +606,13 @@ bool ln_whole_rows(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
 }
-// backward only: rows of up to 4 KiB also fit a block (16 wave-columns), see lds_ln_bwd_wide_shape()
+// forward, fp32 rows of up to 4 KiB: the same kernel with 8 wave-columns and shorter tiles, see lds_ln_4k_shape()
+bool ln_fwd_whole_4k(bool bf16, int C, int K, uintptr_t align_bits) {
+    const long long row_bytes = (long long)C * 4;
+    return !bf16 && lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 2 * kLnCbBytes &&
+           align_bits % 16 == 0;
+}
+// backward: rows of up to 4 KiB also fit a block (16 wave-columns), see lds_ln_bwd_wide_shape()
 bool ln_bwd_whole_4k(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_bwd_wide_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 4096 &&
@@ -705,7 +711,8 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
     hipStream_t s = (hipStream_t)stream;
     const ConvPtrs la{x, nullptr, cu, w, b, y, nullptr};
-    if (ln_wide_rows(bf16, C, K, bits)) {
+    const bool rows4k = ln_fwd_whole_4k(bf16, C, K, bits);
+    if (!rows4k && ln_wide_rows(bf16, C, K, bits)) {
         if (!stats) return -NPLM_DWCONV_ENULL;      // the statistics pass between the two kernels through it
         LdsPlan lp;
         rc = make_default_lds_plan(false, bf16, T, C, K, &lp);
@@ -724,9 +731,9 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
         }
         return -NPLM_DWCONV_EUNSUPPORTED;
     }
-    if (!ln_whole_rows(bf16, C, K, bits)) return -NPLM_DWCONV_EUNSUPPORTED;
+    if (!rows4k && !ln_whole_rows(bf16, C, K, bits)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp{};
-    lp.sh = lds_ln_shape(bf16);
+    lp.sh = rows4k ? lds_ln_4k_shape(bf16, K) : lds_ln_shape(bf16);
     lp.R = lp.sh.rw * lp.sh.nrg;
     lp.ncb = 1;
     lp.ntiles = ceil_div(T, lp.R);
@@ -737,6 +744,15 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     const LnArgs ln{ln_weight, ln_bias, stats, eps};
     const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
     const dim3 grid(lp.nbt);
+    if (rows4k) {
+        switch (K) {
+            case 3: return (int)launch_ln_fwd_4k_k3(bf16, la, ln, g, grid, s);
+            case 5: return (int)launch_ln_fwd_4k_k5(bf16, la, ln, g, grid, s);
+            case 7: return (int)launch_ln_fwd_4k_k7(bf16, la, ln, g, grid, s);
+            case 9: return (int)launch_ln_fwd_4k_k9(bf16, la, ln, g, grid, s);
+        }
+        return -NPLM_DWCONV_EUNSUPPORTED;
+    }
     switch (K) {
         case 3: return (int)launch_ln_fwd_k3(bf16, la, ln, g, grid, s);
         case 5: return (int)launch_ln_fwd_k5(bf16, la, ln, g, grid, s);

@@ -123,6 +123,10 @@ hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, cons
 hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_4k_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_4k_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_4k_k7(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_ln_fwd_4k_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 // LayerNorm-fused backward for rows of one 2 KiB column block (the WHOLE variant of dwconv_bwd_lds_kernel): 8 wave-columns
 // x 4 bytes per lane, 2 row groups of 8 rows (7 at K = 9, where 16 rows of x plus 24 of dy would not fit twice) and no
 // loader waves: all 16 waves compute, each stages its share of the next tile first. Two (dy tile, x tile) pairs =
@@ -230,6 +234,11 @@ constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
 constexpr bool lds_ln_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
 constexpr int kLnCbBytes = 2048;
 constexpr LdsShapeSel lds_ln_shape(bool bf16) { return LdsShapeSel{bf16, bf16 ? 4 : 2, 8, 2, 4, 8, 3}; }
+// fp32 rows of up to 4 KiB (C <= 1024, the residual stream under autocast): 8 wave-columns x 8 bytes per lane and one row
+// group, so that three tiles of at most 13 staged rows fit the LDS (156 KiB): 14 - K rows per tile. Not for bf16 rows of
+// that size (C <= 2048): twice the values per staged row, the loader waves' statistics pass spills at 128 registers and
+// the kernel is slower than the statistics kernel + the normalising conv forward (352 against 303 us at C=2048, K=7).
+constexpr LdsShapeSel lds_ln_4k_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 4 : 2, 14 - K, 1, 8, 8, 3}; }
 constexpr int kLdsDefaultCb = 1024;
 // Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block
 // widths cover the common cases (K <= 9):

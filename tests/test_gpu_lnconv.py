@@ -65,6 +65,36 @@ def test_fused_layernorm_forward_is_deterministic_and_takes_the_boundary_stress_
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize("C", [1024, 644])
+def test_fp32_rows_of_up_to_4_kib_take_the_whole_row_forward_on_the_boundary_stress_mix(C):
+    """The fp32 residual stream (rows of 4 KiB at hidden 1024; 644 channels leave the last wave-columns partly and wholly
+    empty): one kernel, which needs no statistics buffer; a bf16 row of that size goes through the two-kernel path and
+    does need one."""
+    wl = make_workload(5, T=9973, C=C, with_dy=False)
+    g = torch.Generator().manual_seed(C)
+    x = (wl.x.float() * (1 + 3 * torch.rand(wl.T, 1, generator=g)) + torch.randn(wl.T, 1, generator=g))
+    gam = 1 + 0.3 * torch.randn(C, generator=g)
+    bet = 0.2 * torch.randn(C, generator=g)
+    w, b = wl.weight.float(), wl.bias.float()
+    y = _check_fwd(x, wl.cu_seqlens, gam, bet, w, b, f"ln fp32 C={C} boundary stress", residual=True)
+    a = [t.to(DEV) for t in (x, wl.cu_seqlens, gam, bet, w, b)]
+    y2, _ = npa.ln_dwconv_fwd(*a, residual=True)
+    assert torch.equal(y, y2)
+    lib = _lib.load()
+    y3 = torch.empty_like(y2)
+    args = lambda t, o, act: (t.data_ptr(), a[1].data_ptr(), a[2].data_ptr(), a[3].data_ptr(), 1e-5, a[4].data_ptr(), a[5].data_ptr(),
+                              o.data_ptr(), None, wl.T, t.shape[1], wl.K, wl.S, act, 0, 1, None)
+    assert lib.nplm_dwconv_ln_fwd(*args(a[0], y3, 0)) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y3)
+    if C == 1024:
+        xb = torch.cat([a[0], a[0]], 1).bfloat16()          # bf16 rows of 4 KiB
+        gb = torch.cat([a[2], a[2]]); hb = torch.cat([a[3], a[3]]); wb = torch.cat([a[4], a[4]]); bb = torch.cat([a[5], a[5]])
+        rc = lib.nplm_dwconv_ln_fwd(xb.data_ptr(), a[1].data_ptr(), gb.data_ptr(), hb.data_ptr(), 1e-5, wb.data_ptr(), bb.data_ptr(),
+                                    torch.empty_like(xb).data_ptr(), None, wl.T, 2048, wl.K, wl.S, 1, 0, 1, None)
+        assert rc == -1                                      # NPLM_DWCONV_ENULL
+
+
 WIDE = [(torch.bfloat16, torch.bfloat16, 2048), (torch.float32, torch.float32, 1024), (torch.float32, torch.bfloat16, 768),
         (torch.bfloat16, torch.float32, 1536), (torch.float32, torch.float32, 2048), (torch.bfloat16, torch.bfloat16, 1032)]
 
@@ -72,8 +102,9 @@ WIDE = [(torch.bfloat16, torch.bfloat16, 2048), (torch.float32, torch.float32, 1
 @pytest.mark.parametrize("K", [3, 5, 7, 9])
 @pytest.mark.parametrize("dt,wdt,C", WIDE)
 def test_layernorm_forward_of_wide_rows(K, dt, wdt, C):
-    """Rows of more than 2 KiB (up to 8 KiB): the row-statistics kernel, then the conv forward that normalises as it
-    reads: 2, 3, 4, 6 and 8 column blocks, the last one partly filled, rows of 4 and 8 chunks per lane."""
+    """Rows of more than 2 KiB (up to 8 KiB). fp32 rows of up to 4 KiB: the whole-row kernel with 8 wave-columns; the
+    others: the row-statistics kernel, then the conv forward that normalises as it reads: 2, 3, 6 and 8 column blocks,
+    the last one partly filled, rows of 4 and 8 chunks per lane."""
     print(f"[case] ln wide K={K} C={C} {dt} w {wdt}", flush=True)
     _check_fwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C)[:6], f"ln wide K={K} C={C} {dt}")
     _check_fwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False)[:6], f"ln wide residual K={K} C={C} {dt}",
