@@ -8,7 +8,9 @@
 // conv as the sub-module the unfused sequence is LayerNorm (read x, write n), conv (read n, write y), add (read x and
 // y, write): 7 passes over [T, C], of which this kernel keeps 2 (read x, write y) and n is never in memory.
 //
-// A block owns whole rows (C * elemsize <= 2 KiB, one column block), so the row statistics come out of the staged tile.
+// A block owns whole rows (one column block: 2 KiB in 4 wave-columns and 16-row tiles, or, for fp32 rows, 4 KiB in 8
+// wave-columns and tiles of 14 - K rows, see lds_ln_shape() and lds_ln_4k_shape()), so the row statistics come out of
+// the staged tile.
 // Three tile buffers: one being computed, one having its statistics taken, one in flight. A loader wave stages whole
 // rows (rows lw, lw + NWL, ... of a tile), waits by count for its own loads of the tile before the newest one, and takes
 // the statistics of exactly those rows while the compute waves are on the previous tile (a row is 2 x 64 chunks of
@@ -20,7 +22,8 @@
 // the other LDS-staged kernels.
 // Measured (T=131072, C=1024, K=7, bf16, MI355X): 100 us, against 455 us for torch.layer_norm in bf16 + this
 // library's conv + add, and 90 us for the conv alone; the vector ALU is the limit (statistics and normalisation of the
-// K-1 halo rows of every 16-row tile included).
+// K-1 halo rows of every 16-row tile included). fp32, C=1024 (rows of 4 KiB): 226 us against 174 us for the conv alone;
+// there a tile period is as long as its loads take to arrive (13 staged rows per 7 output rows), not the vector ALU.
 //
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); the LayerNorm is
 // torch.nn.LayerNorm's (modeling.py:408-414: eps and bias from the config, 1e-5 and none by default, modeling.py:51-52).
@@ -36,14 +39,6 @@ struct LnArgs {
     float eps;
 };
 
-// Row statistics by the pairwise-combination form of Welford's algorithm (Chan et al.): a lane takes the mean and the
-// sum of squared deviations M2 of its own values exactly (two passes over registers), then the 64 lanes are merged:
-// for two parts of na and nb values,
-//     mean = mean_a + (mean_b - mean_a) * nb / (na + nb),   M2 = M2_a + M2_b + (mean_b - mean_a)^2 * na * nb / (na + nb).
-// No cancellation however far the mean lies from zero. The merge runs in the vector ALU: 4 steps inside each group of
-// 16 lanes by DPP row rotations (8, 4, 2, 1: every lane of a group ends up with the group's result), then the 4 groups'
-// results are read from lanes 0, 16, 32, 48 and merged as wave-uniform values. The counts depend on the lane only
-// (which of its 16-byte chunks lie inside the row), so their factors are set up once.
 // LDS accesses of the loader waves while their direct global->LDS loads of another buffer are in flight: through a
 // volatile address-space-3 pointer. For an ordinary LDS access the compiler first waits for every outstanding vector
 // memory operation (it cannot tell which LDS bytes a direct load will write), which would make the statistics of a

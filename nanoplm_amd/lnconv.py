@@ -8,12 +8,13 @@ For a conv that takes the place of a sub-module of the reference's pre-norm enco
 ``ln_varlen_dwconv(x, cu_seqlens, ln_weight, ln_bias, weight, bias, residual=True)`` returns
 ``x + conv(layer_norm(x))``; the normalised tensor is never stored (K in {3,5,7,9}, rows in multiples of 16 bytes):
 
-* rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32): one kernel, one read of x and one write of y; its blocks
+* rows of at most 2 KiB (C <= 1024 in bf16, 512 in fp32) and fp32 rows of at most 4 KiB (C <= 1024: the residual
+  stream of the reference under ``torch.autocast`` is fp32): one kernel, one read of x and one write of y; its blocks
   own whole rows, take the row statistics from the tile they have staged and normalise as they read;
-* rows of at most 8 KiB (fp32 hidden sizes up to 2048: the residual stream of the reference under ``torch.autocast``
-  is fp32): a row-statistics kernel, then the conv kernel normalising as it reads with the statistics given;
+* other rows of at most 8 KiB: a row-statistics kernel, then the conv kernel normalising as it reads with the
+  statistics given;
 * the forward leaves (mean, rstd) per row for the backward, whose conv kernel normalises x again as it reads it and
-  sums the LayerNorm parameter gradients beside dw and db; for rows of at most 2 KiB its waves also exchange the row
+  sums the LayerNorm parameter gradients beside dw and db; for rows of at most 4 KiB its waves also exchange the row
   sums of the LayerNorm input gradient and write dx themselves (one kernel), for wider rows it hands the gradient of
   the normalised tensor (fp32) to one more pass over the rows.
 
@@ -88,7 +89,7 @@ def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, resid
     (dln_bias None without ``ln_bias``). ``stats`` is the forward's ``[T, 2]`` (mean, rstd).
 
     Fused shapes: the conv backward normalises x as it reads it (the normalised tensor is never stored) and sums the
-    LayerNorm parameter gradients beside dw and db; dx comes from the same kernel (rows of at most 2 KiB) or from one
+    LayerNorm parameter gradients beside dw and db; dx comes from the same kernel (rows of at most 4 KiB) or from one
     more pass over (x, dn, dy). Other shapes compose
     elementwise normalisation in fp32, the plain HIP conv backward and ATen's LayerNorm backward."""
     T, C, K, S = _check(x, cu_seqlens, ln_weight, ln_bias, weight, None)
