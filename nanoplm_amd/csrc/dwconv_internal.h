@@ -133,12 +133,21 @@ hipError_t launch_ln_fwd_4k_k9(bool bf16, const ConvPtrs& p, const LnArgs& ln, c
 // 152 KiB at K = 7, plus 1.3 KiB for the exchange of the row sums and the tiles' row statistics. Measured at T=131072,
 // C=1024, K=7, bf16 (whole call): 8 compute waves of 16 rows + 4 loader waves 271 us (8 loader waves: 497 us, the
 // registers of 16 rows spill at 128 per wave; 12-row waves: 273 us).
-constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 8 : 7, 2, 8, 0, 2}; }
+// fp32 at K <= 7: 4 wave-columns x 8 bytes per lane and 4 row groups of 4 rows instead (T=131072, C=512, K=7: 163 against
+// 178 us per call), as for the 4 KiB rows below.
+constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) {
+    return (!bf16 && K <= 7) ? LdsShapeSel{false, 2, 4, 4, 4, 0, 2} : LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 7 ? 8 : 7, 2, 8, 0, 2};
+}
 // The same for rows of up to 4 KiB (fp32 hidden sizes up to 1024 - the residual stream that torch.autocast leaves - and
-// bf16 up to 2048): 16 wave-columns x 4 bytes per lane, one row group of 8 (K = 3), 6 (K = 5, 7) or 5 (K = 9) rows,
-// 144 KiB of tiles.
+// bf16 up to 2048): tiles of 8 (K = 3), 6 (K = 5, 7) or 5 (K = 9) rows, 144 KiB. bf16, and fp32 at K = 9: 16
+// wave-columns x 4 bytes per lane, one row group. fp32 at K <= 7: 8 wave-columns x 8 bytes per lane, two row groups of
+// 4 or 3 rows - half the LDS reads, stores and exchanged row sums per value (T=131072, C=1024, K=7: 354 against 393 us
+// per call; C=768: 350 against 385 us). In bf16 that split (8 bytes = 4 channels per lane) spills at 128 registers.
 constexpr bool lds_ln_bwd_wide_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
-constexpr LdsShapeSel lds_ln_bwd_wide_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 3 ? 8 : K <= 7 ? 6 : 5, 1, 16, 0, 2}; }
+constexpr LdsShapeSel lds_ln_bwd_wide_shape(bool bf16, int K) {
+    return (!bf16 && K <= 7) ? LdsShapeSel{false, 2, K <= 3 ? 4 : 3, 2, 8, 0, 2}
+                             : LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 3 ? 8 : K <= 7 ? 6 : 5, 1, 16, 0, 2};
+}
 hipError_t launch_ln_bwd_whole4k_k3(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole4k_k5(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_bwd_whole4k_k7(bool bf16, const ConvPtrs& p, const LnSide& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
