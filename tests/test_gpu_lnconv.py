@@ -302,13 +302,18 @@ def test_layernorm_conv_replays_correctly_from_a_hip_graph(dt, C):
             assert torch.equal(a, e), f"replay {it}"
 
 
-def test_layernorm_conv_at_the_headline_size_against_the_composed_ops():
-    """T=131072, C=1024, K=7, bf16 with configuration 3's lengths (8192 tiles, every block 32 rounds): the fused
-    forward and the one-kernel backward against the same operator composed on the GPU in fp32 (torch's LayerNorm, this
-    library's fp32 conv kernels, which the other tests hold to the oracle, ATen's LayerNorm backward): bf16 outputs
-    within one bf16 rounding of the fp32 result where it is not tiny, parameter gradients to 1e-4 of their largest
-    value; and twice the same bits."""
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
+def test_layernorm_conv_at_the_headline_size_against_the_composed_ops(dt):
+    """T=131072, C=1024, K=7 with configuration 3's lengths, in bf16 (8192 tiles, every block 32 rounds) and as the fp32
+    residual stream (rows of 4 KiB: 18725 forward tiles of 7 rows and 21846 backward tiles of 6, the last round partly
+    empty): the fused forward and the one-kernel backward against the same operator composed on the GPU in fp32 (torch's
+    LayerNorm, this library's fp32 conv kernels, which the other tests hold to the oracle, ATen's LayerNorm backward):
+    bf16 outputs within one bf16 rounding of the fp32 result where it is not tiny, fp32 outputs to 1e-4, parameter
+    gradients to 1e-4 of their largest value; and twice the same bits."""
+    import dataclasses
     wl = make_workload(3, with_dy=True)
+    if dt == torch.float32:
+        wl = dataclasses.replace(wl, x=wl.x.float(), dy=wl.dy.float(), dtype=torch.float32)
     d = wl.to(DEV)
     g = torch.Generator().manual_seed(9)
     gam = (1 + 0.3 * torch.randn(wl.C, generator=g)).to(DEV)
@@ -328,9 +333,9 @@ def test_layernorm_conv_at_the_headline_size_against_the_composed_ops():
 
     def act_close(got, ref, what):
         err = (got.float() - ref).abs()
-        bound = ref.abs() * 2.0 ** -8 + 2e-2 * (ref.abs() < 8)
+        bound = ref.abs() * 2.0 ** -8 + 2e-2 * (ref.abs() < 8) if dt == torch.bfloat16 else 1e-4 * (1 + ref.abs())
         bad = int((err > bound).sum())
-        assert bad == 0, f"{what}: {bad} elements beyond one bf16 rounding (max err {float(err.max()):.3e})"
+        assert bad == 0, f"{what}: {bad} elements beyond the bound (max err {float(err.max()):.3e})"
 
     act_close(y, yr.detach(), "y")
     act_close(out[0], xf.grad, "dx")
