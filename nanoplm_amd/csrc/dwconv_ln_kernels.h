@@ -85,18 +85,19 @@ __device__ __forceinline__ float wave_sums4(const float (&v)[4]) {
 // Statistics of NB staged rows of a loader wave (rows lw, lw + nlw, ...): two passes over the wave's registers - the
 // rows' sums, reduced over the wave, give the means; the squared deviations from those means, reduced the same way,
 // the variances - and (rstd, -mean * rstd, mean) per row left in LDS.
-template <typename SH, bool BF16, int NB>
+template <typename SH, bool BF16, int NB, bool FULLROW>
 __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int lw, int nlw, int lane, int C, float eps) {
     static_assert(NB <= 4, "the rows of a loader wave are reduced four at a time");
     constexpr int CE = 16 / SH::E;                        // elements per 16-byte chunk
-    constexpr int NCH = SH::CB_BYTES / 1024;              // chunks per lane and row
+    constexpr int NCHB = SH::CB_BYTES / 1024;             // chunks per lane and row of a full column block
     const int rowb = C * SH::E;
     const float inv_c = 1.f / (float)C;
     float mean[NB], var[NB];
     // straight-line code (all reads first, four partial sums per row) so that the rows' dependency chains overlap; lanes
     // whose chunk lies past the end of a narrow row select zeros
-    auto local = [&](auto full_c) __attribute__((always_inline)) {
+    auto local = [&](auto full_c, auto nch_c) __attribute__((always_inline)) {
         constexpr bool FULL = decltype(full_c)::value;
+        constexpr int NCH = decltype(nch_c)::value;       // chunks per lane and row that hold values of the row
         float v[NB][NCH][CE];
 #pragma unroll
         for (int r = 0; r < NB; ++r) {
@@ -143,7 +144,10 @@ __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int l
 #pragma unroll
         for (int r = 0; r < NB; ++r) var[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(tq), 16 * r)) * inv_c;
     };
-    if (rowb == SH::CB_BYTES) local(std::true_type{}); else local(std::false_type{});
+    // rows that fill the column block, rows one KiB short of it (the last piece is then never staged), anything else
+    if (FULLROW || rowb == SH::CB_BYTES) local(std::true_type{}, std::integral_constant<int, NCHB>{});
+    else if (NCHB > 1 && rowb == SH::CB_BYTES - 1024) local(std::true_type{}, std::integral_constant<int, (NCHB > 1 ? NCHB - 1 : 1)>{});
+    else local(std::false_type{}, std::integral_constant<int, NCHB>{});
 #pragma unroll
     for (int r = 0; r < NB; ++r) {
         const int j = lw + r * nlw;
@@ -154,12 +158,13 @@ __device__ __forceinline__ void ln_stats_pass(const char* buf, float4* st, int l
 
 // Stage rows first_row .. first_row+NROWS-1 (clamped to [0,T)) of `src` into `dst`, whole rows per loader wave: wave
 // lw takes rows lw, lw + nlw, ... with all their 1 KiB pieces, so that its own loads are all it has to wait for
-// before it reads those rows. Every wave issues exactly NB * NPIECE loads with all 64 lanes (a slot past the wave's
-// last row loads that row again; a lane past the end of a narrow row re-reads the row's last 16 bytes into the unused
-// tail of its LDS row), so that "all but the newest tile's loads have landed" is a compile-time s_waitcnt.
+// before it reads those rows. Every wave issues exactly NB * np loads with all 64 lanes, np the number of 1 KiB pieces
+// that hold part of a row (a slot past the wave's last row loads that row again; a lane past the end of a narrow row
+// re-reads the row's last 16 bytes into the unused tail of its piece), so that "all but the newest tile's loads have
+// landed" is an s_waitcnt with one of NPIECE immediates (wait_but_tile). LDS pieces past np are never written.
 template <typename SH, int NB>
 __device__ __forceinline__ void stage_whole_rows(const void* __restrict__ src, char* dst, int first_row, int T, size_t row_bytes,
-                                                 int valid_bytes, int lw, int nlw, int lane) {
+                                                 int valid_bytes, int np, int lw, int nlw, int lane) {
     const int rb = first_row > 0 ? first_row : 0;
     const rsrc_t rs = rows_rsrc(src, rb, T, row_bytes);
     const int rowb = (int)row_bytes;
@@ -171,14 +176,16 @@ __device__ __forceinline__ void stage_whole_rows(const void* __restrict__ src, c
         const bool once = j >= 2 * SH::P && j < SH::NROWS - 2 * SH::P;   // no other tile stages this row
 #pragma unroll
         for (int p = 0; p < SH::NPIECE; ++p) {
-            int boff = p * 1024 + lane * 16;
-            boff = boff < valid_bytes ? boff : valid_bytes - 16;
-            load_to_lds<kLoadAuxOnceFwd>(rs, dst + j * SH::CB_BYTES + p * 1024, boff, so, once);
+            if (p < np) {
+                int boff = p * 1024 + lane * 16;
+                boff = boff < valid_bytes ? boff : valid_bytes - 16;
+                load_to_lds<kLoadAuxOnceFwd>(rs, dst + j * SH::CB_BYTES + p * 1024, boff, so, once);
+            }
         }
     }
 }
 
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL>
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, int NWL, bool FULLROW>
 __global__ void __launch_bounds__((NCW * NRG + NWL) * 64)
 dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu, const void* __restrict__ w,
                      const void* __restrict__ b, void* __restrict__ y, const LnArgs ln, const LdsGeo g) {
@@ -187,7 +194,6 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
     constexpr int BUF_BYTES = SH::TILE_BYTES;
     constexpr int NBUF = 3;     // one tile computed, one having its statistics taken, one in flight
     constexpr int NB = (SH::NROWS + NWL - 1) / NWL;       // staged rows per loader wave
-    constexpr int CNT = NB * SH::NPIECE;                  // loads per loader wave and tile
     using Row = RowVec<BF16, VEC>;
     static_assert(SH::CB_BYTES % 1024 == 0, "whole 1 KiB pieces");
     static_assert(NWL <= SH::NROWS, "every loader wave owns a row");
@@ -205,6 +211,17 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
     const size_t row_bytes = (size_t)C * E;
     const int rowb = (int)row_bytes;
     const int valid_bytes = rowb;                          // <= CB_BYTES (host-checked)
+    // 1 KiB pieces of a staged row that hold part of the row; FULLROW (rows that fill the column block, host-checked)
+    // makes it, the counted wait and the statistics pass compile-time
+    const int np = FULLROW ? SH::NPIECE : (rowb + 1023) >> 10;
+    static_assert(SH::NPIECE <= 4, "wait_but_tile covers up to four pieces per row");
+    // all of this wave's loads but the NB * np of the tile staged last have landed
+    auto wait_but_tile = [&]() __attribute__((always_inline)) {
+        if (np == 1) wait_vmem_but<NB>();
+        else if (np == 2) wait_vmem_but<2 * NB>();
+        else if (np == 3) wait_vmem_but<3 * NB>();
+        else wait_vmem_but<4 * NB>();
+    };
     const int ntl = (g.ntiles + g.nbt - 1) / g.nbt;
 
     const int wc = wv % NCW;
@@ -237,12 +254,12 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
     };
     if (is_loader) {
         const int lw = wv - SH::NWC;
-        stage_whole_rows<SH, NB>(x, lds_raw, tb * R - P, T, row_bytes, valid_bytes, lw, NWL, lane);
+        stage_whole_rows<SH, NB>(x, lds_raw, tb * R - P, T, row_bytes, valid_bytes, np, lw, NWL, lane);
         const int r1 = ntl > 1 ? lds_tile_row0(g, 1, lds_next_slot(g, tb), R) : T;
-        if (r1 < T) stage_whole_rows<SH, NB>(x, lds_raw + BUF_BYTES, r1 - P, T, row_bytes, valid_bytes, lw, NWL, lane);
+        if (r1 < T) stage_whole_rows<SH, NB>(x, lds_raw + BUF_BYTES, r1 - P, T, row_bytes, valid_bytes, np, lw, NWL, lane);
         post_bounds(0, tb * R);
-        if (r1 < T) wait_vmem_but<CNT>(); else wait_vmem_all();       // this wave's rows of tile 0 have landed
-        ln_stats_pass<SH, BF16, NB>(lds_raw, st_all, lw, NWL, lane, C, ln.eps);
+        if (r1 < T) wait_but_tile(); else wait_vmem_all();           // this wave's rows of tile 0 have landed
+        ln_stats_pass<SH, BF16, NB, FULLROW>(lds_raw, st_all, lw, NWL, lane, C, ln.eps);
     } else {
         load_weights<VEC, K>(w, g.w_flags & ~W_RESIDUAL, c0, wr);      // the identity is added from the raw x below
 #pragma unroll
@@ -271,15 +288,15 @@ dwconv_ln_fwd_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu,
             const int lw = wv - SH::NWC;
             const int r1 = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
             const int r2 = it + 2 < ntl ? lds_tile_row0(g, it + 2, lds_next_slot(g, qn), R) : T;
-            if (r2 < T) stage_whole_rows<SH, NB>(x, lds_raw + b2 * BUF_BYTES, r2 - P, T, row_bytes, valid_bytes, lw, NWL, lane);
+            if (r2 < T) stage_whole_rows<SH, NB>(x, lds_raw + b2 * BUF_BYTES, r2 - P, T, row_bytes, valid_bytes, np, lw, NWL, lane);
             if (r1 < T) post_bounds((it + 1) & 1, r1);
             if (r1 < T) {
-                if (r2 < T) wait_vmem_but<CNT>(); else wait_vmem_all();
-                ln_stats_pass<SH, BF16, NB>(lds_raw + b1 * BUF_BYTES, st_all + b1 * SH::NROWS, lw, NWL, lane, C, ln.eps);
+                if (r2 < T) wait_but_tile(); else wait_vmem_all();
+                ln_stats_pass<SH, BF16, NB, FULLROW>(lds_raw + b1 * BUF_BYTES, st_all + b1 * SH::NROWS, lw, NWL, lane, C, ln.eps);
             }
         } else {
             const int tf = t0 + rg * RW;
-            if (tf < T) {
+            if (tf < T && wc * 64 * VEC < C) {          // (a wave-column past the end of a narrow row has nothing to do)
                 {
                     const u32x4 m = *(const volatile __attribute__((address_space(3))) u32x4*)(box + ((it & 1) * NRG + rg) * 16);
                     sc.cs = __builtin_amdgcn_readfirstlane((int)m.x);

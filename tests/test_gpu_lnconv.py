@@ -44,7 +44,8 @@ def _check_fwd(x, cu, gam, bet, w, b, what, residual=False, fused=True):
 @pytest.mark.parametrize("K", [3, 5, 7, 9])
 @pytest.mark.parametrize("dt,wdt,C", [(torch.bfloat16, torch.bfloat16, 1024), (torch.bfloat16, torch.float32, 768),
                                        (torch.float32, torch.float32, 512), (torch.float32, torch.float32, 384),
-                                       (torch.bfloat16, torch.bfloat16, 8), (torch.float32, torch.bfloat16, 100)])
+                                       (torch.bfloat16, torch.bfloat16, 8), (torch.float32, torch.bfloat16, 100),
+                                       (torch.bfloat16, torch.bfloat16, 512)])
 def test_fused_layernorm_forward_kernel_sizes_and_widths(K, dt, wdt, C):
     """Whole rows in one 2 KiB column block: full and partial rows, one chunk per row, both dtypes, mixed
     parameter dtypes; lengths around the 24-row tiles and the 12-row wave windows, empty sequences."""
