@@ -780,7 +780,7 @@ int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
     l.whole4k = ln_bwd_whole_4k(bf16, C, K, 0);
     l.whole = l.whole4k || ln_whole_rows(bf16, C, K, 0);
     if (l.whole) {
-        l.lp.sh = l.whole4k ? lds_ln_bwd_wide_shape(bf16, K) : lds_ln_bwd_shape(bf16, K);
+        l.lp.sh = !l.whole4k ? lds_ln_bwd_shape(bf16, K) : lds_ln_bwd_rows3k(bf16, C) ? lds_ln_bwd_3k_shape(K) : lds_ln_bwd_wide_shape(bf16, K);
         l.lp.R = l.lp.sh.rw * l.lp.sh.nrg;
         l.lp.ncb = 1;
         l.lp.ntiles = ceil_div(T, l.lp.R);

@@ -144,6 +144,11 @@ constexpr LdsShapeSel lds_ln_bwd_shape(bool bf16, int K) {
 // 4 or 3 rows - half the LDS reads, stores and exchanged row sums per value (T=131072, C=1024, K=7: 354 against 393 us
 // per call; C=768: 350 against 385 us). In bf16 that split (8 bytes = 4 channels per lane) spills at 128 registers.
 constexpr bool lds_ln_bwd_wide_kernel_size(int K) { return K == 3 || K == 5 || K == 7 || K == 9; }
+// fp32 rows of 2 to 3 KiB (hidden 768, the reference's default width, modeling.py:42) get a column block of their own:
+// 6 wave-columns x 8 bytes per lane x 2 row groups (12 waves, none without channels) and, the rows being shorter,
+// tiles of 12 (K = 3), 10 (K = 5, 7) or 8 (K = 9) rows in the same LDS.
+constexpr bool lds_ln_bwd_rows3k(bool bf16, long long C) { return !bf16 && C * 4 > 2048 && C * 4 <= 3072; }
+constexpr LdsShapeSel lds_ln_bwd_3k_shape(int K) { return LdsShapeSel{false, 2, K <= 3 ? 6 : K <= 7 ? 5 : 4, 2, 6, 0, 2}; }
 constexpr LdsShapeSel lds_ln_bwd_wide_shape(bool bf16, int K) {
     return (!bf16 && K <= 7) ? LdsShapeSel{false, 2, K <= 3 ? 4 : 3, 2, 8, 0, 2}
                              : LdsShapeSel{bf16, bf16 ? 2 : 1, K <= 3 ? 8 : K <= 7 ? 6 : 5, 1, 16, 0, 2};

@@ -97,7 +97,8 @@ def test_fp32_rows_of_up_to_4_kib_take_the_whole_row_forward_on_the_boundary_str
 
 
 WIDE = [(torch.bfloat16, torch.bfloat16, 2048), (torch.float32, torch.float32, 1024), (torch.float32, torch.bfloat16, 768),
-        (torch.bfloat16, torch.float32, 1536), (torch.float32, torch.float32, 2048), (torch.bfloat16, torch.bfloat16, 1032)]
+        (torch.bfloat16, torch.float32, 1536), (torch.float32, torch.float32, 2048), (torch.bfloat16, torch.bfloat16, 1032),
+        (torch.float32, torch.float32, 644)]
 
 
 @pytest.mark.parametrize("K", [3, 5, 7, 9])
