@@ -733,7 +733,7 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     }
     if (!rows4k && !ln_whole_rows(bf16, C, K, bits)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp{};
-    lp.sh = rows4k ? lds_ln_4k_shape(bf16, K) : lds_ln_shape(bf16);
+    lp.sh = !rows4k ? lds_ln_shape(bf16) : lds_ln_rows3k(bf16, C) ? lds_ln_3k_shape(K) : lds_ln_4k_shape(bf16, K);
     lp.R = lp.sh.rw * lp.sh.nrg;
     lp.ncb = 1;
     lp.ntiles = ceil_div(T, lp.R);

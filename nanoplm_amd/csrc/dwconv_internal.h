@@ -253,6 +253,10 @@ constexpr LdsShapeSel lds_ln_shape(bool bf16) { return LdsShapeSel{bf16, bf16 ? 
 // that size (C <= 2048): twice the values per staged row, the loader waves' statistics pass spills at 128 registers and
 // the kernel is slower than the statistics kernel + the normalising conv forward (352 against 303 us at C=2048, K=7).
 constexpr LdsShapeSel lds_ln_4k_shape(bool bf16, int K) { return LdsShapeSel{bf16, bf16 ? 4 : 2, 14 - K, 1, 8, 8, 3}; }
+// fp32 rows of 2 to 3 KiB (hidden 768): 6 wave-columns and three tiles of 17 staged rows x 3 KiB (18 - K rows per tile),
+// 6 compute + 9 loader waves of two staged rows each.
+constexpr bool lds_ln_rows3k(bool bf16, long long C) { return !bf16 && C * 4 > 2048 && C * 4 <= 3072; }
+constexpr LdsShapeSel lds_ln_3k_shape(int K) { return LdsShapeSel{false, 2, 18 - K, 1, 6, 9, 3}; }
 constexpr int kLdsDefaultCb = 1024;
 // Rows that are not a whole number of 1 KiB column blocks leave the last one partly empty. Three more column-block
 // widths cover the common cases (K <= 9):
