@@ -194,6 +194,9 @@ def main():
     ap.add_argument("--fp32", action="store_true",
                     help="the configuration's tensors in fp32: what a conv on the residual stream receives under "
                          "torch.autocast with fp32 parameters (informational; twice the activation bytes)")
+    ap.add_argument("--channels", type=int, default=None,
+                    help="the configuration's lengths and kernel size at another width, e.g. 768, the reference's default "
+                         "hidden size (informational)")
     ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
     ap.add_argument("--prewarm-ms", type=float, default=1000.0,
                     help="untimed steps run for this long before the warm-up steps")
@@ -219,6 +222,11 @@ def main():
     lib = _lib.load()
 
     wl = make_workload(args.config, with_dy=True)
+    if args.channels and args.channels != wl.C:
+        import dataclasses
+        base_c = wl.C
+        wl = make_workload(args.config, C=args.channels, with_dy=True)
+        wl = dataclasses.replace(wl, name=wl.name.replace(f"_C{base_c}_", f"_C{args.channels}_"))
     if args.fp32 and wl.dtype != torch.float32:
         import dataclasses
         wl = dataclasses.replace(wl, name=wl.name.replace("bf16", "fp32"), dtype=torch.float32, x=wl.x.float(),
@@ -390,7 +398,7 @@ def main():
 
     out = {
         "metric": "varlen dwconv fwd+bwd tokens/s and HBM GB/s (% peak), T=131072 C=1024 K=7 bf16"
-                  if args.config == 3 and not args.gated and not args.ln and not args.fp32 else
+                  if args.config == 3 and not args.gated and not args.ln and not args.fp32 and not args.channels else
                   f"varlen {'gated ' if args.gated else 'layernorm-fused ' if args.ln else ''}dwconv "
                   f"{wl.passes} tokens/s ({wl.name})",
         "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
