@@ -200,10 +200,10 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
  *   dw, db                  the conv's parameter gradients over n = layer_norm(x) (n is recomputed, never stored)
  *   dln_weight, dln_bias    the LayerNorm's parameter gradients, fp32 [C] (dln_bias may be NULL)
  *   dx                      the LayerNorm's input gradient (+ dy with NPLM_DWCONV_RESIDUAL), act_dtype
- * Rows of at most 4 KiB: one kernel (the conv backward normalises x as it
- * reads, its waves exchange the row sums of the LayerNorm input gradient inside the block and write dx) and one small
- * reduction of per-block partial sums. Wider rows: the conv backward writes dn (the gradient of n, fp32) into the workspace and one more pass over (x, dn, dy)
- * rows forms dx. The workspace (nplm_dwconv_ln_bwd_workspace_bytes, 256-byte aligned; 0 for unsupported shapes) holds
+ * Rows of at most 4 KiB: one kernel (the conv backward normalises x as it reads, its waves exchange the row sums of
+ * the LayerNorm input gradient inside the block and write dx) and one small reduction of per-block partial sums.
+ * Wider rows: the conv backward writes dn (the gradient of n, fp32) into the workspace and one more pass over
+ * (x, dn, dy) rows forms dx. The workspace (nplm_dwconv_ln_bwd_workspace_bytes, 256-byte aligned; 0 for unsupported shapes) holds
  * the partial sums and, for the wider rows, dn (T x C x 4 bytes).
  */
 size_t nplm_dwconv_ln_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype);

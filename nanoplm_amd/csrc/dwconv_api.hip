@@ -606,19 +606,21 @@ bool ln_whole_rows(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes <= kLnCbBytes && align_bits % 16 == 0;
 }
-// forward, fp32 rows of up to 4 KiB: the same kernel with 8 wave-columns and shorter tiles, see lds_ln_4k_shape()
+// forward, fp32 rows of up to 4 KiB: the same kernel with 6 or 8 wave-columns and shorter tiles, see lds_ln_3k_shape()
+// and lds_ln_4k_shape()
 bool ln_fwd_whole_4k(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * 4;
     return !bf16 && lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 2 * kLnCbBytes &&
            align_bits % 16 == 0;
 }
-// backward: rows of up to 4 KiB also fit a block (16 wave-columns), see lds_ln_bwd_wide_shape()
+// backward: rows of up to 4 KiB also fit a block, see lds_ln_bwd_wide_shape() and lds_ln_bwd_3k_shape()
 bool ln_bwd_whole_4k(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_bwd_wide_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 4096 &&
            align_bits % 16 == 0;
 }
-// wider rows (up to 8 KiB): a row-statistics kernel, then the conv forward that normalises as it reads
+// other rows of up to 8 KiB: a row-statistics kernel, then the conv forward that normalises as it reads (the forward
+// asks ln_fwd_whole_4k first)
 bool ln_wide_rows(bool bf16, int C, int K, uintptr_t align_bits) {
     const long long row_bytes = (long long)C * (bf16 ? 2 : 4);
     return lds_ln_kernel_size(K) && row_bytes % 16 == 0 && row_bytes > kLnCbBytes && row_bytes <= 8192 && align_bits % 16 == 0;
