@@ -66,11 +66,12 @@ def test_fused_layernorm_forward_is_deterministic_and_takes_the_boundary_stress_
     assert torch.equal(y, y2)
 
 
-@pytest.mark.parametrize("C", [1024, 644])
+@pytest.mark.parametrize("C", [1024, 644, 516, 772])
 def test_fp32_rows_of_up_to_4_kib_take_the_whole_row_forward_on_the_boundary_stress_mix(C):
-    """The fp32 residual stream (rows of 4 KiB at hidden 1024; 644 channels leave the last wave-columns partly and wholly
-    empty): one kernel, which needs no statistics buffer; a bf16 row of that size goes through the two-kernel path and
-    does need one."""
+    """The fp32 residual stream (rows of 4 KiB at hidden 1024; 644 channels leave the last wave-columns of the 3 KiB
+    column block partly and wholly empty; 516 and 772 channels put 16 bytes into the last 1 KiB piece of the 3 KiB and
+    the 4 KiB block): one kernel, which needs no statistics buffer; a bf16 row of that size goes through the two-kernel
+    path and does need one."""
     wl = make_workload(5, T=9973, C=C, with_dy=False)
     g = torch.Generator().manual_seed(C)
     x = (wl.x.float() * (1 + 3 * torch.rand(wl.T, 1, generator=g)) + torch.randn(wl.T, 1, generator=g))
@@ -98,7 +99,7 @@ def test_fp32_rows_of_up_to_4_kib_take_the_whole_row_forward_on_the_boundary_str
 
 WIDE = [(torch.bfloat16, torch.bfloat16, 2048), (torch.float32, torch.float32, 1024), (torch.float32, torch.bfloat16, 768),
         (torch.bfloat16, torch.float32, 1536), (torch.float32, torch.float32, 2048), (torch.bfloat16, torch.bfloat16, 1032),
-        (torch.float32, torch.float32, 644)]
+        (torch.float32, torch.float32, 644), (torch.float32, torch.bfloat16, 516), (torch.float32, torch.float32, 772)]
 
 
 @pytest.mark.parametrize("K", [3, 5, 7, 9])
@@ -116,8 +117,9 @@ def test_layernorm_forward_of_wide_rows(K, dt, wdt, C):
 @pytest.mark.parametrize("K", [3, 7, 9])
 @pytest.mark.parametrize("dt,wdt,C", WIDE)
 def test_layernorm_backward_of_wide_rows(K, dt, wdt, C):
-    """Rows of more than 2 KiB: the one-kernel backward with 16 wave-columns (up to 4 KiB) and the two-kernel path
-    (conv backward leaving the normalised tensor's gradient in fp32, then the row pass for dx)."""
+    """Rows of more than 2 KiB: the one-kernel backward (up to 4 KiB: 16 wave-columns of 4 bytes per lane, or, in fp32,
+    8 or 6 wave-columns of 8 bytes in two row groups) and the two-kernel path (conv backward leaving the normalised
+    tensor's gradient in fp32, then the row pass for dx)."""
     print(f"[case] ln bwd wide K={K} C={C} {dt} w {wdt}", flush=True)
     _check_bwd(*_case(LENS_MIX, C, K, dt, wdt, seed=K + C), f"ln bwd wide K={K} C={C} {dt}")
     _check_bwd(*_case(LENS_MIX[::-1], C, K, dt, wdt, seed=K + C + 1, ln_bias=False), f"ln bwd wide residual K={K} C={C} {dt}",
