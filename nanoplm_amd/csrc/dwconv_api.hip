@@ -741,6 +741,10 @@ int nplm_dwconv_ln_fwd(const void* x, const int32_t* cu, const void* ln_weight, 
     lp.ntiles = ceil_div(T, lp.R);
     lp.nbt = lp.ntiles < kNumCU ? lp.ntiles : kNumCU;          // one block of 16 waves and three tiles per CU
     lp.xcd_group = (lp.nbt % (kNumXCD * 8) == 0) ? 8 : 0;
+    // fp32 rows of 4 KiB: 6 of a tile's 13 staged rows are a neighbour's, and a neighbour on another XCD means reading them
+    // from HBM again; 32 consecutive tiles per XCD instead of 8 (T=131072, C=1024, K=7: 217 against 222 us per call; the
+    // other whole-row kernels, with longer tiles, measure the same either way)
+    if (rows4k && lp.nbt % (kNumXCD * 32) == 0) lp.xcd_group = 32;
     lp.rot_step = lp.nbt > 2 ? (int)((long long)lp.nbt * 618 / 1000) | 1 : 0;
     if (lp.rot_step >= lp.nbt) lp.rot_step = lp.nbt - 1;
     const LnArgs ln{ln_weight, ln_bias, stats, eps};
