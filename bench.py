@@ -44,6 +44,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E
+VALU_PEAK_TFLOPS = 157.3  # MI355X fp32 vector ALU (256 CUs x 4 SIMDs x 32 FMA lanes x 2 flop x 2.4 GHz)
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and
 # scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
@@ -117,6 +118,10 @@ def cpu_baseline(wl, sample_tokens):
     n = max(1, min(n, cu.numel() - 1))
     Ts = int(cu[n])
     x, dy, cus = wl.x[:Ts], wl.dy[:Ts], cu[: n + 1]
+    # every host core the box gives this process (BASELINE: torch.set_num_threads(os.cpu_count())); both counts are reported
+    threads_default = torch.get_num_threads()
+    host_cores = os.cpu_count() or threads_default
+    torch.set_num_threads(host_cores)
     threads = torch.get_num_threads()
 
     def run(dtype):
@@ -136,6 +141,7 @@ def cpu_baseline(wl, sample_tokens):
                   f"torch conv1d + autograd in {str(wl.dtype).replace('torch.', '')}, median of 3 after 1 warm-up",
         "seconds_per_pass": t_bf16,
         "fp32_tokens_per_s": Ts / t_f32,
+        "os_cpu_count": host_cores, "torch_default_threads": threads_default,
     }
 
 
@@ -176,6 +182,94 @@ def device_loop_baseline(d, passes, reps=3):
             "sequences": len(cu) - 1, "what": f"per-sequence torch conv1d loop + autograd on the GPU, {passes}"}
 
 
+def autograd_step_times(npa, d, xs, gs, args, nset):
+    """The step as a model pays for it: ``VarlenDWConv1d`` forward + ``y.backward(dy)`` (the call site a conv module
+    has in the reference: src/nanoplm/pretraining/models/modern_bert/modeling.py:421-439, backward driven by
+    src/nanoplm/pretraining/pure_pipeline.py:739-742), on the same rotating tensor sets and in the same order as the
+    raw loop: the backward of a step runs two forwards after its own forward. One block = nset steps
+    (F0 F1 F2 B0 F3 B1 B2 B3). Timed eagerly (host work of the wrappers included; it overlaps the GPU as long as it is
+    shorter) and replayed from one captured HIP graph of a block. Gradients are set to None before every block, as
+    ``optimizer.zero_grad(set_to_none=True)`` does, so nothing is accumulated into an old gradient."""
+    import torch
+
+    wl_dtype = d.x.dtype
+    T, C = d.x.shape
+    K = d.weight.shape[1]
+    dev = d.x.device
+    conv = npa.VarlenDWConv1d(C, K, residual=bool(args.residual or args.ln)).to(dev).to(d.weight.dtype)
+    with torch.no_grad():
+        conv.weight.copy_(d.weight)
+        conv.bias.copy_(d.bias)
+    norm = None
+    if args.ln:
+        norm = torch.nn.LayerNorm(C, eps=1e-5).to(dev).to(d.weight.dtype)
+    cu = d.cu_seqlens
+    leaves = [x.detach().requires_grad_(True) for x in xs]
+    params = list(conv.parameters()) + (list(norm.parameters()) if norm is not None else [])
+
+    def forward(j):
+        if args.ln:
+            return conv.forward_prenorm(leaves[j], cu, norm)
+        if args.gated:
+            return conv.forward_gated(leaves[j], cu)
+        return conv(leaves[j], cu)
+
+    def block():
+        for t in leaves + params:
+            t.grad = None
+        ys = []
+        for j in range(nset):
+            ys.append(forward(j))
+            if j >= 2:
+                ys[j - 2].backward(gs[j - 2])
+        for j in range(nset - 2, nset):
+            ys[j].backward(gs[j])
+
+    def timed(fn, nblocks, reps):
+        out = []
+        for _ in range(reps):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(nblocks):
+                fn()
+            torch.cuda.synchronize()
+            out.append((time.perf_counter() - t0) * 1e3 / (nblocks * nset))
+        return out
+
+    nblocks = max(1, (args.steps + nset - 1) // nset)
+    for _ in range(max(2, args.warmup // nset)):
+        block()
+    eager = timed(block, nblocks, max(1, args.reps))
+    res = {"ms_per_step_autograd": statistics.median(eager), "ms_per_step_autograd_min": min(eager),
+           "autograd_what": f"VarlenDWConv1d{'.forward_prenorm' if args.ln else '.forward_gated' if args.gated else ''} + "
+                            f"y.backward(dy), blocks of {nset} steps on the rotating sets, eager"}
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                block()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for t in leaves + params:
+            t.grad = None
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            block()
+        graph.replay()
+        torch.cuda.synchronize()
+        rep = timed(graph.replay, nblocks, max(1, args.reps))
+        res["ms_per_step_autograd_graph"] = statistics.median(rep)
+        res["ms_per_step_autograd_graph_min"] = min(rep)
+        del graph
+    except Exception as exc:      # a capture that fails must not lose the rest of the line
+        res["ms_per_step_autograd_graph"] = None
+        res["autograd_graph_error"] = f"{type(exc).__name__}: {exc}"[:300]
+    for t in leaves + params:
+        t.grad = None
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -198,12 +292,14 @@ def main():
                     help="the configuration's lengths and kernel size at another width, e.g. 768, the reference's default "
                          "hidden size (informational)")
     ap.add_argument("--reps", type=int, default=15, help="repetitions of the timed K-step loop (median reported)")
-    ap.add_argument("--prewarm-ms", type=float, default=1000.0,
+    ap.add_argument("--prewarm-ms", type=float, default=6000.0,
                     help="untimed steps run for this long before the warm-up steps")
     ap.add_argument("--device-loop", action="store_true",
                     help="also time the per-sequence torch conv1d loop (the reference's way to this op) on the GPU; "
                          "its first pass can take minutes while the convolution library prepares kernels per length")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-autograd", action="store_true",
+                    help="skip the module-level figures (ms_per_step_autograd, ms_per_step_autograd_graph)")
     ap.add_argument("--cpu-sample-tokens", type=int, default=65536)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -335,6 +431,11 @@ def main():
             torch.cuda.synchronize()
             same_ms.append((time.perf_counter() - t0) * 1e3 / args.steps)
 
+    # ---- the same step through the module and autograd (the surface a model calls), eagerly and from a HIP graph ----
+    autograd = None
+    if fwd_bwd and not args.no_autograd:
+        autograd = autograd_step_times(npa, d, xs, gs, args, NSET)
+
     # ---- per-kernel durations with HIP events on the launch stream ---------------------------------
     # The same step sequence as the timed loop above, launched back to back without host
     # synchronisation, with one pair of events per step around the kernel being measured; one pass
@@ -384,11 +485,25 @@ def main():
     step_bytes = fwd_bytes + bwd_bytes
 
     def roof(nbytes, samples_us, kernel):
+        """Roofline of one kernel against both ceilings it can meet: HBM on its algorithmic bytes and the fp32 vector
+        ALU on its algorithmic flops (forward 2KTC, backward 4KTC + TC; no MFMA in this op). `bound` names the ceiling
+        that takes longer at its peak, i.e. the one that binds; achieved/peak/unit/frac are that ceiling's, and both
+        ceilings' figures are kept under "hbm" and "valu"."""
         med = statistics.median(samples_us)
         gbps = nbytes / med / 1e3
+        flops = wl.algorithmic_flops("fwd" if kernel == "forward" else "bwd")
+        tflops = flops / med / 1e6
         traffic = (MEASURED_TRAFFIC.get((wl.name, kernel, "ln")) if args.ln else
                    None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel)))
-        r = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+        hbm = {"achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+               "algorithmic_bytes": nbytes, "us_at_peak": nbytes / HBM_PEAK_GBPS / 1e3}
+        valu = {"achieved": tflops, "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / VALU_PEAK_TFLOPS,
+                "algorithmic_flops": flops, "us_at_peak": flops / VALU_PEAK_TFLOPS / 1e6}
+        valu_bound = valu["us_at_peak"] >= hbm["us_at_peak"] and not (args.gated or args.ln)
+        top = valu if valu_bound else hbm
+        r = {"bound": "valu" if valu_bound else "hbm", "achieved": top["achieved"], "peak": top["peak"], "unit": top["unit"],
+             "frac": top["frac"], "flops_per_byte": flops / nbytes, "ridge_flops_per_byte": VALU_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBPS,
+             "hbm": hbm, "valu": valu,
              "traffic": traffic, "kernel": kernel, "median_us": med, "min_us": min(samples_us),
              "avg_us": statistics.fmean(samples_us), "launches": len(samples_us), "algorithmic_bytes": nbytes}
         if traffic is None:
@@ -413,7 +528,15 @@ def main():
         "step_algorithmic_bytes": step_bytes,
         "step_GBps": step_bytes / (ms_per_step * 1e-3) / 1e9,
         "step_frac_of_hbm_peak": step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "step_algorithmic_flops": wl.algorithmic_flops(),
+        "step_TFLOPps": wl.algorithmic_flops() / (ms_per_step * 1e-3) / 1e12,
+        "step_frac_of_valu_peak": wl.algorithmic_flops() / (ms_per_step * 1e-3) / 1e12 / VALU_PEAK_TFLOPS,
     }
+    if autograd:
+        out.update(autograd)
+        out["autograd_over_raw"] = autograd["ms_per_step_autograd"] / ms_per_step
+        out["autograd_graph_over_raw"] = (autograd["ms_per_step_autograd_graph"] / ms_per_step
+                                          if autograd.get("ms_per_step_autograd_graph") else None)
     if fwd_bwd:
         out["roofline"] = roof(bwd_bytes, bwd_us, "backward")
         out["roofline_fwd"] = roof(fwd_bytes, fwd_us, "forward")

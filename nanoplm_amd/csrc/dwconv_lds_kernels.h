@@ -461,14 +461,17 @@ dwconv_fwd_lds_kernel(const void* __restrict__ x, const int32_t* __restrict__ cu
             // one dword per lane: lane l of a load takes float l of the tile's [NROWS][2] statistics (rows clamped like
             // the tile's own)
             if (wv == SH::NWC) {
-                const rsrc_t rst = make_rsrc(ln.stats, (uint32_t)T * 8u);
+                // descriptor based at the tile's first row (like the tile's own), so that the lane offsets stay small
+                // whatever T is
+                const int sb = first_row > 0 ? first_row : 0;
+                const rsrc_t rst = rows_rsrc(ln.stats, sb, T, 8);
                 char* d = st_base + (buf == lds_raw ? 0 : ST_BYTES);
 #pragma unroll
                 for (int l0 = 0; l0 < SH::NROWS * 2; l0 += 64) {
                     const int idx = l0 + lane;
                     if (idx < SH::NROWS * 2)
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rst, (lds_void*)(d + l0 * 4), 4, (clamp_row(first_row + idx / 2, T) * 2 + (idx & 1)) * 4,
-                                                                 0, 0, kLoadAux);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(rst, (lds_void*)(d + l0 * 4), 4,
+                                                                 ((clamp_row(first_row + idx / 2, T) - sb) * 2 + (idx & 1)) * 4, 0, 0, kLoadAux);
                 }
             }
         }
@@ -1163,7 +1166,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     }
                     s1 *= inv_c;
                     s2 *= -inv_c;
-                    // straight-line for all rows: the stores of rows past the end fall outside dx's buffer range
+                    // straight-line arithmetic for all rows; only the store of a row past the end is skipped
 #pragma unroll
                     for (int u = 0; u < RW; ++u) {
                         {
@@ -1179,7 +1182,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                                 o[v] = __builtin_fmaf(rstd, __builtin_fmaf(nm2, xh[u][v], __builtin_fmaf(gam[v], dnv[u][v], -m1)), o[v]);
                             Row orow;
                             orow.from_f32(o);
-                            if (active) orow.bstore(ro, out_voff, u * rowb);
+                            if (active && tf + u < T) orow.bstore(ro, out_voff, u * rowb);
                         }
                     }
                 }

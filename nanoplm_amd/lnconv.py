@@ -50,16 +50,26 @@ def _check(x, cu_seqlens, ln_weight, ln_bias, weight, bias):
     return T, C, weight.shape[1], cu_seqlens.numel() - 1
 
 
+def _param_dtype(weight, ln_weight, ln_bias):
+    """The one dtype the kernels take every parameter in: the conv weight's when the LayerNorm parameters share it,
+    else fp32 (the wider of the two; casting the other way would round the fp32 parameters to bf16)."""
+    for t in (ln_weight, ln_bias):
+        if t is not None and t.dtype != weight.dtype:
+            return torch.float32
+    return weight.dtype
+
+
 def ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: float = 1e-5, residual: bool = False,
                   want_stats: bool = True):
     """Raw forward (no autograd): ``(y, stats)`` with y = conv(layer_norm(x)) (+ x) in x's dtype and stats
-    ``[T, 2]`` fp32 = (mean, rstd) per row (None without ``want_stats``). The LayerNorm parameters are used in the
-    conv weight's dtype."""
+    ``[T, 2]`` fp32 = (mean, rstd) per row (None without ``want_stats``). The kernels take the LayerNorm parameters
+    and the conv parameters in one dtype: when they differ (fp32 ``nn.LayerNorm`` parameters beside bf16 taps, say), all
+    of them go in as fp32 for this call, so that no parameter is rounded."""
     T, C, K, S = _check(x, cu_seqlens, ln_weight, ln_bias, weight, bias)
     lib = _lib.load()
     x = x.contiguous()
-    weight = weight.contiguous()
-    wdt = weight.dtype
+    wdt = _param_dtype(weight, ln_weight, ln_bias)
+    weight = weight.to(wdt).contiguous()
     ln_weight = ln_weight.to(wdt).contiguous()
     ln_bias = None if ln_bias is None else ln_bias.to(wdt).contiguous()
     bias = None if bias is None else bias.to(wdt).contiguous()
@@ -101,8 +111,8 @@ def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, resid
     x = x.contiguous()
     dy = dy.contiguous()
     stats = stats.contiguous()
-    weight = weight.contiguous()
-    wdt = weight.dtype
+    wdt = _param_dtype(weight, ln_weight, ln_bias)
+    weight = weight.to(wdt).contiguous()
     lnw = ln_weight.to(wdt).contiguous()
     lnb = None if ln_bias is None else ln_bias.to(wdt).contiguous()
     act = _DTYPES[x.dtype]

@@ -52,6 +52,14 @@ class Workload:
         passes = passes or self.passes
         return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[passes]
 
+    def algorithmic_flops(self, passes: Optional[str] = None) -> int:
+        """Floating-point operations one launch must do: fwd = 2KTC; bwd = 4KTC (dx and dw) + TC (db)."""
+        T, C, K = self.T, self.C, self.K
+        fwd = 2 * K * T * C
+        bwd = 4 * K * T * C + T * C
+        passes = passes or self.passes
+        return {"fwd": fwd, "bwd": bwd, "fwd+bwd": fwd + bwd}[passes]
+
 
 _SPECS = {
     1: dict(name="cfg1_fp32_fwd_8seq_C64_K3", passes="fwd", dtype=torch.float32, T=None, C=64, K=3, mix="n8_u20_128"),

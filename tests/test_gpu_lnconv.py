@@ -187,6 +187,19 @@ def test_fused_layernorm_backward_kernel_sizes_and_widths(K, dt, wdt, C):
                residual=True)
 
 
+@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.bfloat16, 2048), (torch.float32, 768)])
+def test_fp32_layernorm_parameters_beside_bf16_taps_are_not_rounded(dt, C):
+    """nn.LayerNorm keeps fp32 parameters under autocast while the conv's taps may be bf16 (FSDP mixed precision):
+    every parameter then goes into the kernels as fp32, so the result is that of the fp32 LayerNorm parameters (an
+    oracle run with gamma and beta rounded to bf16 differs from it by more than the tolerance on d ln_weight)."""
+    x, cu, gam, bet, w, b, dy = _case(LENS_MIX, C, 7, dt, torch.bfloat16, seed=C + 3)
+    g = torch.Generator().manual_seed(C)
+    gam = 1 + 0.3 * torch.randn(C, generator=g)          # fp32, not representable in bf16
+    bet = 0.2 * torch.randn(C, generator=g)
+    _check_fwd(x, cu, gam, bet, w, b, f"mixed ln dtypes C={C} {dt}", residual=True)
+    _check_bwd(x, cu, gam, bet, w, b, dy, f"mixed ln dtypes bwd C={C} {dt}", residual=True)
+
+
 def test_fused_layernorm_backward_is_deterministic_and_takes_the_boundary_stress_mix():
     wl = make_workload(5, T=20011, C=1024, with_dy=True)        # lengths of 1..8 mixed with 400..512, odd T
     g = torch.Generator().manual_seed(6)

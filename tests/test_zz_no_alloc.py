@@ -5,6 +5,8 @@ Both run the same kernels on the same launch geometry, so every output must be b
 made through the C ABI (ctypes), two in a row on the same GPU with the second one smaller, so that
 whatever the first call left in the shared array is there when the second one runs.
 """
+import ctypes
+
 import pytest
 import torch
 
@@ -13,6 +15,21 @@ from nanoplm_amd.workloads import cu_from_lengths, make_workload
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
+
+
+_hip = None
+
+
+def _device_free_bytes():
+    """Free device memory as the HIP runtime counts it (hipMemGetInfo through ctypes)."""
+    global _hip
+    if _hip is None:
+        _hip = ctypes.CDLL("libamdhip64.so")
+        _hip.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    rc = _hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total))
+    assert rc == 0, f"hipMemGetInfo failed: {rc}"
+    return free.value
 
 
 def _inputs(lens, C, K, dt, seed):
@@ -49,13 +66,24 @@ def _bwd_pair(x, dy, cu, w, flags=0, want_dx=True, want_red=True):
     ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=DEV)
     _lib.check(lib.nplm_dwconv_bwd_ex(p(x), p(dy), p(cu), p(w), p(ref[0]), p(ref[1]), p(ref[2]), p(ws), ws.numel(),
                                       T, C, K, S, act, wdt, flags, stream), "nplm_dwconv_bwd_ex")
+    def static(o):
+        _lib.check(lib.nplm_dwconv_bwd_static(p(x), p(dy), p(cu), p(w), p(o[0]), p(o[1]), p(o[2]),
+                                              T, C, K, S, act, wdt, flags, stream), "nplm_dwconv_bwd_static")
+
+    # first call on this shape: may look up the scratch address and raise a kernel's LDS limit (no allocation either,
+    # but the runtime may load a code object); the call that is bracketed below is a warm one
+    static(outs())
     got = outs()
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
-    _lib.check(lib.nplm_dwconv_bwd_static(p(x), p(dy), p(cu), p(w), p(got[0]), p(got[1]), p(got[2]),
-                                          T, C, K, S, act, wdt, flags, stream), "nplm_dwconv_bwd_static")
+    free_before = _device_free_bytes()
+    static(got)
+    # the device's own count of free memory (hipMemGetInfo) sees a hipMalloc/hipFree inside the library, which torch's
+    # caching allocator cannot; read it again while the call's kernels may still be running and after they have ended
+    assert _device_free_bytes() == free_before, "nplm_dwconv_bwd_static changed the device's free memory"
     assert torch.cuda.memory_allocated() == before
     torch.cuda.synchronize()
+    assert _device_free_bytes() == free_before, "nplm_dwconv_bwd_static changed the device's free memory"
     return ref, got
 
 
@@ -132,3 +160,42 @@ def test_empty_batch_zero_fills():
     assert rc == 0
     torch.cuda.synchronize()
     assert float(dw.abs().max()) == 0.0 and float(db.abs().max()) == 0.0
+
+
+def test_static_backward_is_captured_and_replayed_by_a_hip_graph():
+    """The callers the entry point is for: a HIP graph capture, under which an allocation inside the call would fail
+    the capture. Captured once (after a warm call outside the capture), replayed with new contents in the static input
+    buffers, with eager work and synchronisation between the replays; every replay equals nplm_dwconv_bwd_ex."""
+    lib = _lib.load()
+    x, dy, cu, w = _inputs([100, 3, 512, 1, 408, 2, 2, 77], 1024, 7, torch.bfloat16, 11)
+    T, C = x.shape
+    K, S = w.shape[1], cu.numel() - 1
+    dx = torch.empty_like(x)
+    dw = torch.empty((C, K), dtype=torch.float32, device=DEV)
+    db = torch.empty((C,), dtype=torch.float32, device=DEV)
+
+    def call():
+        _lib.check(lib.nplm_dwconv_bwd_static(x.data_ptr(), dy.data_ptr(), cu.data_ptr(), w.data_ptr(), dx.data_ptr(),
+                                              dw.data_ptr(), db.data_ptr(), T, C, K, S, _lib.BF16, _lib.BF16, 0,
+                                              torch.cuda.current_stream().cuda_stream), "nplm_dwconv_bwd_static")
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                                         # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for it in range(3):
+        nx, ndy, _, _ = _inputs([100, 3, 512, 1, 408, 2, 2, 77], 1024, 7, torch.bfloat16, 20 + it)
+        x.copy_(nx)
+        dy.copy_(ndy)
+        dx.fill_(float("nan"))
+        dw.fill_(float("nan"))
+        db.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, _ = _bwd_pair(nx, ndy, cu, w)
+        assert torch.equal(dx, ref[0]) and torch.equal(dw, ref[1]) and torch.equal(db, ref[2]), f"replay {it}"
