@@ -68,6 +68,7 @@ extern "C" {
 
 /* flags of the _ex entry points */
 #define NPLM_DWCONV_RESIDUAL 1u   /* fuse the residual connection: y = x + conv(x), dx = dy + conv^T(dy) */
+#define NPLM_DWCONV_GRADS_BF16 2u /* nplm_dwconv_bwd_ex / _static only: dw and db point to bf16 buffers */
 
 #define NPLM_DWCONV_MAX_K 255
 
@@ -122,7 +123,11 @@ int nplm_dwconv_bwd(const void* x, const void* dy, const int32_t* cu, const void
 /*
  * Backward with flags. With NPLM_DWCONV_RESIDUAL, dx = dy + conv^T(dy; w) (the gradient of
  * x + conv(x) with respect to x); dw and db are those of the convolution and do not change.
- * flags == 0 is nplm_dwconv_bwd.
+ * With NPLM_DWCONV_GRADS_BF16, dw and db are bf16 buffers ([C,K] and [C], 2-byte aligned, passed
+ * through the float* parameters): the sums are still formed in fp32 in the same fixed order and are
+ * rounded once, nearest-even, as they are stored, which is what casting the fp32 results gives; it
+ * saves a bf16 parameter's gradient the two cast kernels (autograd hands a parameter a gradient
+ * of its own dtype: FSDP2 bf16 parameters, pure_pipeline.py:483-487). flags == 0 is nplm_dwconv_bwd.
  */
 int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const void* w,
                        void* dx, float* dw, float* db, void* workspace, size_t workspace_bytes,

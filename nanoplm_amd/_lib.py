@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(_HERE, "libnplm_dwconv.so")
 F32 = 0
 BF16 = 1
 RESIDUAL = 1    # NPLM_DWCONV_RESIDUAL
+GRADS_BF16 = 2  # NPLM_DWCONV_GRADS_BF16
 EUNSUPPORTED = 10   # NPLM_DWCONV_EUNSUPPORTED
 ESCRATCH = 11       # NPLM_DWCONV_ESCRATCH
 STATIC_SCRATCH_BYTES = 16 << 20   # NPLM_DWCONV_STATIC_SCRATCH_BYTES

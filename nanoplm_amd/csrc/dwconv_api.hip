@@ -343,6 +343,15 @@ __global__ void fill_zero_kernel(float* p, long long n) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0.f;
 }
+__global__ void fill_zero16_kernel(uint16_t* p, long long n) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+hipError_t fill_zero16(void* p, long long n, hipStream_t s) {
+    if (!p || n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(fill_zero16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, (uint16_t*)p, n);
+    return hipGetLastError();
+}
 hipError_t fill_zero(float* p, long long n, hipStream_t s) {
     if (!p || n <= 0) return hipSuccess;
     hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, p, n);
@@ -434,13 +443,14 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
              int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream, const nplm_dwconv_tuning* tune) {
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
-    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    if (flags & ~(uint32_t)(NPLM_DWCONV_RESIDUAL | NPLM_DWCONV_GRADS_BF16)) return -NPLM_DWCONV_EFLAGS;
     const int w_flags = kernel_w_flags(w_dtype, flags);
+    const int out_bf16 = (flags & NPLM_DWCONV_GRADS_BF16) ? 1 : 0;      // dw, db are bf16 buffers
     hipStream_t s = (hipStream_t)stream;
     const bool want_red = dw || db;
     if (T == 0) {
-        hipError_t e = fill_zero(dw, (long long)C * K, s);
-        if (e == hipSuccess) e = fill_zero(db, C, s);
+        hipError_t e = out_bf16 ? fill_zero16(dw, (long long)C * K, s) : fill_zero(dw, (long long)C * K, s);
+        if (e == hipSuccess) e = out_bf16 ? fill_zero16(db, C, s) : fill_zero(db, C, s);
         return (int)e;
     }
     if (!dx && !want_red) return 0;
@@ -450,7 +460,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx;
     if (bits % E) return -NPLM_DWCONV_EALIGN;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
-    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
+    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % (out_bf16 ? 2 : 4)) return -NPLM_DWCONV_EALIGN;
 
     int algo = choose_algo(true, tune, bf16, T, C, K, bits);
     if (algo < 0) return algo;
@@ -477,7 +487,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         }
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0,
-                           s, (const float*)part, lp.nbt, C, K, dw, db);
+                           s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
         return (int)hipGetLastError();
     }
     if (algo == 2) {
@@ -503,7 +513,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         if (want_red) {
             const long long n_out = (long long)(K + 1) * C;
             hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)),
-                               dim3(64 * FIN_SPLIT), 0, s, (const float*)part, lp.nbt, C, K, dw, db);
+                               dim3(64 * FIN_SPLIT), 0, s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
             e = hipGetLastError();
         }
         return (int)e;
@@ -568,7 +578,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     if (want_red) {
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)partial, p.nbt, C, K, dw, db);
+                           (const float*)partial, p.nbt, C, K, dw, db, out_bf16);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
@@ -941,7 +951,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, p.nbt, C, K, dw, db);
+                           (const float*)part, p.nbt, C, K, dw, db, 0);
         return (int)hipGetLastError();
     }
     if (!gated_supported(true, bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
@@ -966,7 +976,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     if (e != hipSuccess) return (int)e;
     const long long n_out = (long long)(K + 1) * C;
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, lp.nbt, C, K, dw, db);
+                       (const float*)part, lp.nbt, C, K, dw, db, 0);
     return (int)hipGetLastError();
 }
 

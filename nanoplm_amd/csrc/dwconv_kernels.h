@@ -423,7 +423,9 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
                                         for (int v = 0; v < VEC; ++v) {
                                             const float gv = ok ? gw[RG::slot(ph, u + m)][v] : 0.f;
                                             if constexpr (WDX) acc[v] = __builtin_fmaf(wr[v][K - 1 - m], gv, acc[v]);
-                                            if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(xc[u][v], gv, dwa[v][K - 1 - m]);
+                                            // x is selected too: an Inf or NaN in this row times the selected zero
+                                            // would put a NaN into a tap sum the product does not belong to
+                                            if constexpr (WDW) dwa[v][K - 1 - m] = __builtin_fmaf(ok ? xc[u][v] : 0.f, gv, dwa[v][K - 1 - m]);
                                         }
                                     }
                                     if constexpr (GATED) {
@@ -494,9 +496,10 @@ dwconv_bwd_kernel(const void* __restrict__ x, const void* __restrict__ dy, const
 constexpr int FIN_SPLIT = 16;
 
 // One block of the reduction: 64 consecutive (tap, channel) outputs, SPLIT groups of slabs summed in LDS.
+// out_bf16: dw and db are bf16 buffers (the fp32 totals are rounded once, nearest-even, on store).
 template <int SPLIT>
 __device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int block, const float* __restrict__ partial, int nbt, int C,
-                                               int K, float* __restrict__ dw, float* __restrict__ db) {
+                                               int K, float* __restrict__ dw, float* __restrict__ db, int out_bf16 = 0) {
     const int lane = (int)(threadIdx.x & 63);
     const int grp = (int)(threadIdx.x >> 6);
     const long long n_out = (long long)(K + 1) * C;
@@ -527,16 +530,21 @@ __device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int bloc
         for (int g = 1; g < SPLIT; ++g) tot += red[g][lane];
         const int kk = (int)(o / C);
         const int c = (int)(o - (long long)kk * C);
-        if (kk < K) { if (dw) dw[(size_t)c * K + kk] = tot; }
-        else        { if (db) db[c] = tot; }
+        if (out_bf16) {
+            if (kk < K) { if (dw) reinterpret_cast<uint16_t*>(dw)[(size_t)c * K + kk] = f32_to_bf16(tot); }
+            else        { if (db) reinterpret_cast<uint16_t*>(db)[c] = f32_to_bf16(tot); }
+        } else {
+            if (kk < K) { if (dw) dw[(size_t)c * K + kk] = tot; }
+            else        { if (db) db[c] = tot; }
+        }
     }
 }
 
 template <int SPLIT>
 __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
-                                                                     float* __restrict__ dw, float* __restrict__ db) {
+                                                                     float* __restrict__ dw, float* __restrict__ db, int out_bf16) {
     __shared__ float red[SPLIT][64];
-    finalize_block<SPLIT>(red, (int)blockIdx.x, partial, nbt, C, K, dw, db);
+    finalize_block<SPLIT>(red, (int)blockIdx.x, partial, nbt, C, K, dw, db, out_bf16);
 }
 
 // Two slab sets of the same launch in one reduction launch (the conv's dw/db and, as a conv of K2 = 1 tap, the

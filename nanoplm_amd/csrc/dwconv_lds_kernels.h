@@ -864,6 +864,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
             // WHOLE: dn of the wave's rows, kept across the exchange of the row sums; (mean, rstd) of the tile's rows
             float dnv[WHOLE ? RW : 1][VEC], xh[WHOLE ? RW : 1][VEC];       // ... and their normalised x
             bool located = false;       // WHOLE: the next tile's boundary lookup has been done (see emit_dx)
+            bool fix_dw = false;        // boundary path: some x value of the wave's rows is Inf or NaN (see xbad there)
             const float2* stl = reinterpret_cast<const float2*>(lds_raw + 2 * BUF_BYTES + RED_BYTES) + (it & 1) * R;
             if (tf < T) {
                 const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
@@ -1085,9 +1086,27 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     uint32_t vm[RW];
                     wave_tap_masks<RW, K>(sc, nce, cuq, S, T, tf, vm);
                     float xc[WDW ? RW : 1][VEC];
+                    // A masked tap enters the dw sums as x * (selected 0), which is NaN for an x that is Inf or NaN,
+                    // where the definition drops the product. Such x values are rare enough to be handled apart: the
+                    // wave tests its x rows (x * 0 summed up is NaN iff one of them is not finite), and if any is, the
+                    // values in question run through the schedule as zeros and add_nonfinite_x below puts their
+                    // valid products into the sums afterwards.
+                    bool xbad = false;
                     if constexpr (WDW) {
 #pragma unroll
                         for (int u = 0; u < RW; ++u) read_x(u, xc[u]);
+                        float chk = 0.f;
+#pragma unroll
+                        for (int u = 0; u < RW; ++u)
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) chk = __builtin_fmaf(xc[u][v], 0.f, chk);
+                        xbad = __builtin_amdgcn_ballot_w64(chk != chk) != 0;
+                        if (xbad) {
+#pragma unroll
+                            for (int u = 0; u < RW; ++u)
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) xc[u][v] = __builtin_isfinite(xc[u][v]) ? xc[u][v] : 0.f;
+                        }
                     }
                     float acc[WDX ? RW : 1][VEC];
                     if constexpr (WDX) {
@@ -1141,6 +1160,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         }
                     }
                     emit_dx(acc);
+                    fix_dw = xbad;
                 }
             }
             if constexpr (WHOLE) {
@@ -1184,6 +1204,56 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                             orow.from_f32(o);
                             if (active && tf + u < T) orow.bstore(ro, out_voff, u * rowb);
                         }
+                    }
+                }
+            }
+            // Boundary path, x rows that hold Inf or NaN (see xbad there): the products of those values with the dy rows
+            // of their own sequence, one output row at a time, once everything else of the tile is done (the tile stays
+            // in LDS until the barrier below). A rolled loop over the rows (their LDS addresses are formed at run time),
+            // the taps unrolled, each behind a scalar branch on its bit of the row's tap mask; lanes whose x value is
+            // finite keep their sums (their products went through the schedule).
+            if constexpr (WDW) {
+                if (fix_dw) {
+                    const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
+                    const char* lpg = cur + loff;
+                    const char* lpx = cur + SH::TILE_BYTES + loff;
+                    SeqCursor sq = sc;
+                    bool fresh = true;
+#pragma nounroll
+                    for (int u = 0; u < RW; ++u) {
+                        const int t = tf + u;
+                        if (t >= T) break;
+                        advance_prefetched(sq, nce, fresh, cuq, S, T, t);
+                        const uint32_t m = row_tap_mask<K>(sq, t);
+                        float xv[VEC];
+                        if constexpr (GATED) {
+                            float uu[VEC], gg[VEC];
+                            lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, uu);
+                            lds_row<SELF, BF16, VEC>(lpx + XT_BYTES + u * SH::CB_BYTES, gg);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) xv[v] = gate_mul(uu[v], gg[v]);
+                        } else {
+                            lds_row<SELF, BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                            if constexpr (NORM) {
+                                const float mean = ln.stats[2 * (size_t)t], rstd = ln.stats[2 * (size_t)t + 1];
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v)
+                                    xv[v] = __builtin_fmaf(__builtin_fmaf(xv[v], rstd, -mean * rstd), gam[v], bet[v]);
+                            }
+                        }
+                        bool nf[VEC];
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) nf[v] = !__builtin_isfinite(xv[v]);
+                        static_for<K>([&](auto kk_c) {
+                            constexpr int kk = decltype(kk_c)::value;
+                            if ((m >> kk) & 1u) {
+                                float gr[VEC];
+                                lds_row<SELF, BF16, VEC>(lpg + (u + kk) * SH::CB_BYTES, gr);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v)
+                                    dwa[v][K - 1 - kk] = nf[v] ? __builtin_fmaf(xv[v], gr[v], dwa[v][K - 1 - kk]) : dwa[v][K - 1 - kk];
+                            }
+                        });
                     }
                 }
             }

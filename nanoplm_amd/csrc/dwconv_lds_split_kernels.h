@@ -400,11 +400,70 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                     }
                 }
             } else {
+                // The passes below mask by multiplying with zeros (x rows of other sequences are zeroed, dy rows of other
+                // sequences are zeroed in the conversion), which turns an Inf or NaN on the other side into a NaN in a
+                // tap sum the product does not belong to. A boundary wave therefore first tests the rows it is about to
+                // use (the sum of their squares is finite iff all of them are; a finite value beyond 1e19 overflows it
+                // and merely takes the slow path too) and, if any is not finite, forms its sums one output row at a
+                // time with every product behind a scalar branch: same products, same order, nothing multiplied by 0.
+                bool exact = false;
+                if (!interior) {
+                    float chk = 0.f;
+                    auto add_sq = [&](const Row& r) __attribute__((always_inline)) {
+                        if constexpr (BF16 && VEC == 2) {
+                            const bf16x2 pr = __builtin_bit_cast(bf16x2, r.d[0]);
+                            chk = __builtin_amdgcn_fdot2_f32_bf16(pr, pr, chk, false);
+                        } else {
+                            float f[VEC];
+                            r.to_f32(f);
+#pragma unroll
+                            for (int v = 0; v < VEC; ++v) chk = __builtin_fmaf(f[v], f[v], chk);
+                        }
+                    };
+                    static_for<NJ>([&](auto j_c) __attribute__((always_inline)) {
+                        Row r;
+                        r.load(lpi + decltype(j_c)::value * SH::CB_BYTES);
+                        add_sq(r);
+                    });
+                    static_for<RW>([&](auto u_c) __attribute__((always_inline)) {
+                        Row r;
+                        r.load(lpx + decltype(u_c)::value * SH::CB_BYTES);
+                        add_sq(r);
+                    });
+                    exact = __builtin_amdgcn_ballot_w64(!__builtin_isfinite(chk)) != 0;
+                }
+                if (exact) {
+                    SeqCursor sq = sc;
+                    bool fresh = true;
+#pragma nounroll
+                    for (int u = 0; u < RW; ++u) {
+                        const int t = tf + u;
+                        if (t >= T) break;
+                        advance_prefetched(sq, nce, fresh, cu, S, T, t);
+                        int jlo = sq.cs - (tf - P), jhi = sq.ce - (tf - P);      // staged rows of row t's sequence
+                        jlo = __builtin_amdgcn_readfirstlane(jlo < 0 ? 0 : jlo);
+                        jhi = __builtin_amdgcn_readfirstlane(jhi > NJ ? NJ : jhi);
+                        float xv[VEC], gc[VEC];
+                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                        lds_read_row<BF16, VEC>(lpi + (u + P) * SH::CB_BYTES, gc);
+#pragma unroll
+                        for (int v = 0; v < VEC; ++v) c[v] += gc[v];
+                        static_for<K>([&](auto m_c) __attribute__((always_inline)) {
+                            constexpr int m = decltype(m_c)::value;
+                            if (u + m >= jlo && u + m < jhi) {
+                                float gr[VEC];
+                                lds_read_row<BF16, VEC>(lpi + (u + m) * SH::CB_BYTES, gr);
+#pragma unroll
+                                for (int v = 0; v < VEC; ++v) a[v][m] = __builtin_fmaf(xv[v], gr[v], a[v][m]);
+                            }
+                        });
+                    }
+                }
                 // one code path for interior and boundary tiles (two regions that both update the K tap sums make the
                 // register allocator keep them twice): one pass per sequence that owns output rows of the wave; an
                 // interior tile is the single pass over all rows
                 SeqCursor sq = sc;
-                int u0 = 0;
+                int u0 = exact ? RW : 0;
                 bool fresh = true;
                 while (u0 < RW && tf + u0 < T) {
                     int jlo = 0, jhi = NJ, u1 = RW;

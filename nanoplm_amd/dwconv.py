@@ -121,10 +121,13 @@ def bwd_workspace_bytes(T: int, C: int, K: int, dtype: torch.dtype) -> int:
 
 
 def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, residual: bool = False,
-                      tuning: Optional[_lib.Tuning] = None, workspace: Optional[torch.Tensor] = None):
+                      tuning: Optional[_lib.Tuning] = None, workspace: Optional[torch.Tensor] = None,
+                      grads_bf16: bool = False):
     """(dx, dw, db): dx in x's dtype (or None), dw [C,K] and db [C] in fp32 (or None, None).
 
-    With ``residual`` dx is the gradient of x + conv(x), i.e. dy + conv^T(dy); dw and db do not change."""
+    With ``residual`` dx is the gradient of x + conv(x), i.e. dy + conv^T(dy); dw and db do not change.
+    With ``grads_bf16`` dw and db come back in bf16: the same fp32 sums, rounded once by the kernel that forms them
+    (what ``dw.to(torch.bfloat16)`` would give, without the two cast kernels)."""
     T, C, K, S = _validate(x, cu_seqlens, weight, None)
     if dy.shape != x.shape or dy.dtype != x.dtype or dy.device != x.device:
         raise ValueError("dy must match x in shape, dtype and device")
@@ -135,8 +138,9 @@ def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, 
     cu_seqlens = cu_seqlens.contiguous()
     act = _DTYPES[x.dtype]
     dx = torch.empty_like(x) if need_dx else None
-    dw = torch.empty((C, K), dtype=torch.float32, device=x.device) if need_dw else None
-    db = torch.empty((C,), dtype=torch.float32, device=x.device) if need_dw else None
+    gdt = torch.bfloat16 if grads_bf16 else torch.float32
+    dw = torch.empty((C, K), dtype=gdt, device=x.device) if need_dw else None
+    db = torch.empty((C,), dtype=gdt, device=x.device) if need_dw else None
     with _launch_on(x) as dev:
         if need_dw and workspace is None:
             if tuning is None:
@@ -145,7 +149,7 @@ def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, 
                 nbytes = int(lib.nplm_dwconv_bwd_slabs(T, C, K, act, tuning)) * (K + 1) * C * 4
             workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
         stream = dev.stream
-        flags = _lib.RESIDUAL if residual else 0
+        flags = (_lib.RESIDUAL if residual else 0) | (_lib.GRADS_BF16 if grads_bf16 else 0)
         args = (_ptr(x), _ptr(dy), _ptr(cu_seqlens), _ptr(weight), _ptr(dx), _ptr(dw), _ptr(db),
                 _ptr(workspace), 0 if workspace is None else workspace.numel() * workspace.element_size(),
                 T, C, K, S, act, _DTYPES[weight.dtype])
@@ -190,8 +194,10 @@ class VarlenDWConv1dFunction(torch.autograd.Function):
         need_dw = ctx.needs_input_grad[2] or (ctx.bias_dtype is not None and ctx.needs_input_grad[3])
         if dy.dtype != x.dtype:
             dy = dy.to(x.dtype)
+        # bf16 parameters take their gradients in bf16 straight from the reduction kernel (no cast kernels)
+        grads_bf16 = weight.dtype == torch.bfloat16 and ctx.bias_dtype in (None, torch.bfloat16)
         dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, need_dx=need_dx, need_dw=need_dw,
-                                       residual=ctx.residual)
+                                       residual=ctx.residual, grads_bf16=grads_bf16)
         if dw is not None:
             dw = dw.to(weight.dtype) if ctx.needs_input_grad[2] else None
             db = db.to(ctx.bias_dtype) if (ctx.bias_dtype is not None and ctx.needs_input_grad[3]) else None
@@ -319,17 +325,18 @@ def _(x, cu_seqlens, weight, bias, residual=False):
 
 @torch.library.custom_op("nanoplm_amd::varlen_dwconv_bwd", mutates_args=(), device_types="cuda")
 def varlen_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
-                         residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(dx, dw, db) with dw [C,K] and db [C] in fp32."""
-    dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, residual=residual)
+                         residual: bool = False, grads_bf16: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dx, dw, db) with dw [C,K] and db [C] in fp32 (bf16 with ``grads_bf16``)."""
+    dx, dw, db = varlen_dwconv_bwd(x, dy, cu_seqlens, weight, residual=residual, grads_bf16=grads_bf16)
     return dx, dw, db
 
 
 @varlen_dwconv_bwd_op.register_fake
-def _(x, dy, cu_seqlens, weight, residual=False):
+def _(x, dy, cu_seqlens, weight, residual=False, grads_bf16=False):
     C, K = weight.shape
+    gdt = torch.bfloat16 if grads_bf16 else torch.float32
     return (torch.empty_like(x, memory_format=torch.contiguous_format),
-            x.new_empty((C, K), dtype=torch.float32), x.new_empty((C,), dtype=torch.float32))
+            x.new_empty((C, K), dtype=gdt), x.new_empty((C,), dtype=gdt))
 
 
 def _op_setup_context(ctx, inputs, output):
@@ -343,7 +350,8 @@ def _op_backward(ctx, dy):
     x, cu_seqlens, weight = ctx.saved_tensors
     if dy.dtype != x.dtype:
         dy = dy.to(x.dtype)
-    dx, dw, db = varlen_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, weight, ctx.residual)
+    grads_bf16 = weight.dtype == torch.bfloat16 and ctx.bias_dtype in (None, torch.bfloat16)
+    dx, dw, db = varlen_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, weight, ctx.residual, grads_bf16)
     return dx, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype)), None
 
 

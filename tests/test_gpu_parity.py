@@ -63,6 +63,63 @@ def test_configuration_1_against_the_fp32_reference_path():
     assert rel <= 1e-5, rel
 
 
+def _elementwise_rel(got, ref64, floor=1e-3):
+    """Largest |got - ref| / |ref| over the elements with |ref| > floor (below it the quotient measures cancellation
+    among the K products of size ~1, not the implementation)."""
+    err = (got.detach().cpu().double() - ref64).abs()
+    big = ref64.abs() > floor
+    return float((err[big] / ref64[big].abs()).max()) if big.any() else 0.0
+
+
+@pytest.mark.parametrize("name,index,kw", [("cfg1", 1, {}), ("cfg3_fp32_T8192_C1024", 3, dict(T=8192, C=1024))])
+def test_fp32_elementwise_error_is_that_of_the_fp32_reference_path(name, index, kw):
+    """"1e-5 relative" for fp32 is met norm-wise (max error / max |ref|, see gpu_util.assert_act_close). Element by
+    element no fp32 evaluation meets it where the taps cancel; the reference path itself (per-sequence torch conv1d +
+    autograd in fp32, oracle/dwconv_ref.py) does not. The bar here: against the same float64 oracle, the kernels' largest
+    element-wise relative error is at most twice the fp32 reference path's own (plus 1e-6), for every output."""
+    wl = make_workload(index, with_dy=True, **kw)
+    x, w, b, dy, cu = wl.x.float(), wl.weight.float(), wl.bias.float(), wl.dy.float(), wl.cu_seqlens
+    y64 = O.c_oracle_fwd(x, cu, w, b)
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
+    ref = O.ref_dwconv_varlen_grads(x, cu, w, b, dy, torch.float32)
+    xd, wd, bd, dyd, cud = (t.to(DEV) for t in (x, w, b, dy, cu))
+    y = npa.varlen_dwconv_fwd(xd, cud, wd, bd)
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    stats = {}
+    for what, got, r32, r64 in (("y", y, ref[0], y64), ("dx", dx, ref[1], dx64), ("dw", dw, ref[2], dw64), ("db", db, ref[3], db64)):
+        k_rel, r_rel = _elementwise_rel(got, r64), _elementwise_rel(r32, r64)
+        k_norm = float((got.cpu().double() - r64).abs().max() / r64.abs().max())
+        r_norm = float((r32.double() - r64).abs().max() / r64.abs().max())
+        stats[what] = {"kernel_max_rel": k_rel, "fp32_reference_path_max_rel": r_rel, "kernel_normwise": k_norm,
+                       "fp32_reference_path_normwise": r_norm}
+        print(f"[parity] {name} fp32 {what}: element-wise max-rel kernel {k_rel:.3e}, fp32 reference path {r_rel:.3e}; "
+              f"norm-wise kernel {k_norm:.3e}, reference path {r_norm:.3e}", flush=True)
+        assert k_rel <= 2.0 * r_rel + 1e-6, f"{name} {what}: kernel {k_rel:.3e} vs fp32 reference path {r_rel:.3e}"
+        assert k_norm <= 1e-5
+    record_parity(f"fp32_elementwise_{name}", {"workload": wl.name, "T": wl.T, "C": wl.C, "K": wl.K, **stats})
+
+
+@pytest.mark.parametrize("C,K,dt", [(1024, 7, torch.bfloat16), (2048, 31, torch.bfloat16), (256, 5, torch.bfloat16),
+                                     (100, 11, torch.float32), (768, 15, torch.bfloat16)])
+def test_parameter_gradients_straight_in_bf16(C, K, dt):
+    """NPLM_DWCONV_GRADS_BF16: the reduction kernel stores dw and db as bf16, rounding its fp32 totals once; that is bit
+    for bit the cast of the fp32 outputs (every kernel family ends in the same reduction kernel). dx is unaffected."""
+    x, cu, w, b, dy = _random_case([33, 1, 200, 2, 90, 64, 63, 7], C, K, dt, torch.bfloat16, seed=C * K)
+    xd, cud, wd, dyd = (t.to(DEV) for t in (x, cu, w, dy))
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    dx2, dw2, db2 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, grads_bf16=True)
+    assert dw2.dtype == torch.bfloat16 and db2.dtype == torch.bfloat16
+    assert torch.equal(dx, dx2) and torch.equal(dw.bfloat16(), dw2) and torch.equal(db.bfloat16(), db2)
+    # a request for dw/db alone may take another kernel family (other summation order): against its own fp32 result
+    _, dw3, db3 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False, grads_bf16=True, residual=True)
+    _, dw4, db4 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False, residual=True)
+    assert torch.equal(dw3, dw4.bfloat16()) and torch.equal(db3, db4.bfloat16())
+    # empty batch: zero-filled in bf16
+    e = torch.empty((0, C), dtype=dt, device=DEV)
+    _, dw0, db0 = npa.varlen_dwconv_bwd(e, e, torch.zeros(1, dtype=torch.int32, device=DEV), wd, grads_bf16=True)
+    assert dw0.dtype == torch.bfloat16 and float(dw0.float().abs().max()) == 0.0 and float(db0.float().abs().max()) == 0.0
+
+
 # ---- golden vectors -------------------------------------------------------------------------------
 @pytest.mark.parametrize("name", ["cfg1_fp32_C64_K3", "boundary_fp32_C16_K7", "stress_bf16_C32_K7"])
 def test_golden_vectors(name, golden_dir):
@@ -189,6 +246,61 @@ def test_nothing_leaks_across_sequences_even_nan_and_inf():
         assert torch.equal(y0[keep], y2[keep]), f"forward leaked out of sequence {seq}"
         assert torch.equal(dx0[keep], dx2[keep]), f"dx leaked out of sequence {seq}"
         assert bool(torch.isnan(y2[s:e]).all())
+
+
+# lengths with sequences of one and two rows in the middle of tiles, next to tile edges and at the very end (the last
+# tile is partial, so its waves also hold copies of the last row)
+POISON_LENS = [40, 1, 2, 50, 1, 300, 2, 30, 7, 1, 213, 2, 64, 1, 33, 700, 2, 1]
+
+
+def _poison_rows(cul, lens, which):
+    """Rows of the sequences picked by ``which`` = [(index into lens, ...)] -> (slice list, set of |k - P| reached)."""
+    rows, reach = [], 0
+    for i in which:
+        rows.append((cul[i], cul[i + 1]))
+        reach = max(reach, lens[i] - 1)
+    return rows, reach
+
+
+@pytest.mark.parametrize("C,K,dt", [(1024, 7, torch.bfloat16), (1024, 7, torch.float32), (256, 7, torch.bfloat16),
+                                     (768, 9, torch.bfloat16), (2048, 31, torch.bfloat16), (1024, 15, torch.bfloat16),
+                                     (512, 31, torch.float32), (104, 11, torch.bfloat16), (1024, 3, torch.bfloat16)])
+def test_nonfinite_rows_reach_only_the_taps_their_products_belong_to(C, K, dt):
+    """dw[c, k] sums x[t + k - P] * dy[t] over the pairs of rows that lie in one sequence. A sequence of L rows
+    therefore contributes to the taps with |k - P| < L only: an Inf or NaN in it makes those taps non-finite and must
+    leave every other tap of dw (and db, when only x is poisoned) exactly as it is without the poison, on the
+    boundary paths of every kernel family (LDS-staged, sliding-window, role-split, runtime-K). Checked against the
+    clean run (bit-equal on the untouched taps) and against the oracle (same finite set, same values there)."""
+    print(f"[case] non-finite rows and dw: C={C} K={K} {dt}", flush=True)
+    P = (K - 1) // 2
+    x, cu, w, b, dy = _random_case(POISON_LENS, C, K, dt, dt, seed=C + K)
+    cul = cu.tolist()
+    xd, cud, wd, dyd = (t.to(DEV) for t in (x, cu, w, dy))
+    _, dw0, db0 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    ones = [i for i, n in enumerate(POISON_LENS) if n == 1]
+    twos = [i for i, n in enumerate(POISON_LENS) if n == 2]
+    cases = [("x: Inf in every one-row sequence", ones, float("inf"), True),
+             ("x: NaN in every two-row sequence", twos, float("nan"), True),
+             ("x: Inf in the last row of the batch", [len(POISON_LENS) - 1], float("-inf"), True),
+             ("dy: Inf in every one-row sequence", ones, float("inf"), False),
+             ("dy: NaN in a two-row sequence", twos[1:2], float("nan"), False)]
+    for what, which, val, in_x in cases:
+        rows, reach = _poison_rows(cul, POISON_LENS, which)
+        x2, dy2 = x.clone(), dy.clone()
+        for s, e in rows:
+            (x2 if in_x else dy2)[s:e] = val
+        _, dw, db = npa.varlen_dwconv_bwd(x2.to(DEV), dy2.to(DEV), cud, wd)
+        dw64, db64 = O.c_oracle_bwd(x2, dy2, cu, w)[1:]
+        touched = torch.tensor([abs(k - P) <= reach for k in range(K)])
+        assert bool((~torch.isfinite(dw[:, touched])).all()), f"{what}: a tap the rows feed stayed finite"
+        assert torch.equal(dw[:, ~touched], dw0[:, ~touched]), f"{what}: a tap the rows do not feed changed"
+        assert torch.equal(torch.isfinite(dw).cpu(), torch.isfinite(dw64)), f"{what}: finite set differs from the oracle's"
+        if (~touched).any():
+            assert_red_close(dw[:, ~touched], dw64[:, ~touched], f"{what}: dw")
+        if in_x:
+            assert torch.equal(db, db0), f"{what}: db changed"
+        else:
+            assert bool((~torch.isfinite(db)).all()) and bool((~torch.isfinite(db64)).all())
 
 
 def test_static_packed_cu_seqlens():

@@ -241,7 +241,8 @@ def test_custom_ops_trace_with_fake_tensors():
     assert str(torch.ops.nanoplm_amd.varlen_dwconv_fwd.default._schema) == (
         "nanoplm_amd::varlen_dwconv_fwd(Tensor x, Tensor cu_seqlens, Tensor weight, Tensor? bias, bool residual=False) -> Tensor")
     assert str(torch.ops.nanoplm_amd.varlen_dwconv_bwd.default._schema) == (
-        "nanoplm_amd::varlen_dwconv_bwd(Tensor x, Tensor dy, Tensor cu_seqlens, Tensor weight, bool residual=False) -> (Tensor, Tensor, Tensor)")
+        "nanoplm_amd::varlen_dwconv_bwd(Tensor x, Tensor dy, Tensor cu_seqlens, Tensor weight, bool residual=False, bool grads_bf16=False) -> "
+        "(Tensor, Tensor, Tensor)")
     with FakeTensorMode():
         x = torch.empty(100, 64, dtype=torch.bfloat16, device="cuda")
         cu = torch.empty(5, dtype=torch.int32, device="cuda")
