@@ -279,16 +279,17 @@ bool split_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) 
     const SplitShapeSel sh = lds_split_shape(false, bf16, K);      // the column block is the same in both passes
     return (long long)C * E >= (long long)sh.ncw * 64 * sh.vec * E;
 }
-int make_split_plan(bool fwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out) {
+int make_split_plan(bool fwd, bool bf16, long long T, int C, int K, const nplm_dwconv_tuning* tune, LdsPlan* out,
+                    bool gated = false) {
     LdsPlan p{};
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    const SplitShapeSel sh = lds_split_shape(fwd, bf16, K);
+    const SplitShapeSel sh = gated ? lds_split_gated_shape(bf16, K) : lds_split_shape(fwd, bf16, K);
     const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
     const long long row_bytes = (long long)C * E;
     p.R = sh.rw * sh.nrg;
-    if ((long long)(p.R + K) * row_bytes + 2 * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
+    if ((long long)(p.R + K) * row_bytes * (gated ? 2 : 1) + 2 * row_bytes >= INT_MAX) return -NPLM_DWCONV_ESHAPE;
     p.ncb = ceil_div(row_bytes, cb_bytes);
     p.ntiles = ceil_div(T, p.R);
     int nbt = tune->nbt > 0 ? tune->nbt : kNumCU / p.ncb;     // one block of 16 waves per CU
@@ -367,7 +368,14 @@ bool gated_supported(bool bwd, bool bf16, long long T, int C, int K, uintptr_t a
     return (long long)C * E >= 1024;
 }
 
-// Long gated backward (K = 15, 31): the sliding-window kernel with one channel per lane; same shapes as the gated forward.
+// Long gated backward (K = 15, 31), role-split (dwconv_lds_split_kernels.h, GATED): rows of whole 16-byte chunks that fill
+// at least one 512-byte column block, 16-byte aligned tensors. Measured at T=131072, C=2048, bf16, backward + finalize
+// against the sliding-window kernel below (log-normal length mix / one long sequence): K=31 728 / 685 against 949 / 808 us,
+// K=15 584 / 535 against 613 / 593 us; dz is the same bit for bit (same tap order).
+bool split_gated_eligible(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
+    return split_eligible(bf16, T, C, K, align_bits);
+}
+// Otherwise: the sliding-window kernel with one channel per lane; same shapes as the gated forward.
 bool long_gated_bwd_supported(bool bf16, long long T, int C, int K, uintptr_t align_bits) {
     return long_gated_kernel_size(K) && gated_supported(false, bf16, T, C, K, align_bits);
 }
@@ -906,9 +914,14 @@ size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, in
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     if (long_gated_bwd_supported(bf16, T, C, K, 0)) {
+        // enough for either kernel: which one runs also depends on pointer alignment, not known here
         Plan p;
         if (make_long_gated_plan(bf16, T, C, K, &p)) return 0;
-        const size_t bytes = (size_t)p.nbt * (K + 1) * C * sizeof(float);
+        int slabs = p.nbt;
+        LdsPlan lp;
+        if (split_gated_eligible(bf16, T, C, K, 0) && make_split_plan(false, bf16, T, C, K, nullptr, &lp, true) == 0 && lp.nbt > slabs)
+            slabs = lp.nbt;
+        const size_t bytes = (size_t)slabs * (K + 1) * C * sizeof(float);
         return (bytes + 255) & ~(size_t)255;
     }
     if (!gated_supported(true, bf16, T, C, K, 0)) return 0;
@@ -935,6 +948,23 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
+    if (long_gated_kernel_size(K) && split_gated_eligible(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
+        LdsPlan lp;
+        rc = make_split_plan(false, bf16, T, C, K, nullptr, &lp, true);
+        if (rc) return rc;
+        const size_t slab = (size_t)(K + 1) * C * sizeof(float);
+        if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab * (size_t)lp.nbt) return -NPLM_DWCONV_EWORKSPACE;
+        float* part = reinterpret_cast<float*>(workspace);
+        const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+        const dim3 grid(lp.ncb * lp.nbt);
+        hipError_t e = K == 31 ? launch_bwd_split_gated_k31(bf16, la, lg, grid, s) : launch_bwd_split_gated_k15(bf16, la, lg, grid, s);
+        if (e != hipSuccess) return (int)e;
+        const long long n_out = (long long)(K + 1) * C;
+        hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
+                           (const float*)part, lp.nbt, C, K, dw, db, 0);
+        return (int)hipGetLastError();
+    }
     if (long_gated_bwd_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
         Plan p;
         rc = make_long_gated_plan(bf16, T, C, K, &p);

@@ -106,7 +106,7 @@ NPLM_DECLARE_LDS_GATED_K(5)
 NPLM_DECLARE_LDS_GATED_K(7)
 NPLM_DECLARE_LDS_GATED_K(9)
 #undef NPLM_DECLARE_LDS_GATED_K
-// long gated kernels: sliding-window fused backward with one channel per lane,
+// long gated kernels: sliding-window fused backward with one channel per lane (rows the role-split kernel does not take),
 hipError_t launch_bwd_gated_k15(bool bf16, int unroll, int maxt, const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block,
                                 size_t shmem, hipStream_t s);
 hipError_t launch_bwd_gated_k31(bool bf16, int unroll, int maxt, const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block,
@@ -118,6 +118,9 @@ hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, c
 hipError_t launch_bwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_bwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+// gated role-split backward (z = [u | g] in, dz out), see lds_split_gated_shape()
+hipError_t launch_bwd_split_gated_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_bwd_split_gated_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 // LayerNorm-fused forward (dwconv_ln_kernels.h), K <= 9, fixed shape per dtype, see lds_ln_shape()
 hipError_t launch_ln_fwd_k3(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_ln_fwd_k5(bool bf16, const ConvPtrs& p, const LnArgs& ln, const LdsGeo& g, dim3 grid, hipStream_t s);
@@ -240,6 +243,15 @@ constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
     (void)K;
     return SplitShapeSel{bf16 ? 2 : 1, 16, fwd ? 8 : 4, 2};
 }
+// Gated role-split backward (K = 31, 15): a buffer holds a u tile and a g tile behind the dy tile, so the tiles are
+// shorter: two buffers of (R + K-1) + 2 R rows of 512 bytes fit the LDS with 4 row groups of 10 rows at K = 31
+// (154 KiB) and of 12 rows at K = 15 (158 KiB).
+// Measured at T=131072, C=2048, K=31, bf16 (backward + finalize, log-normal mix / one long sequence): 728 / 685 us;
+// 256-byte column blocks with 8 row groups of 12 rows (96-row tiles) 721 / 673; 8 rows per wave 776 / 720; one channel
+// per lane in 256-byte blocks with 16, 20, 24 rows per wave 784 / 732, 765 / 718, 771 / 702: rows per wave count, tile
+// length does not. Both roles evaluate the gate's sigmoid (two quarter-rate instructions per element and role),
+// which is what the kernel costs over the plain one (510 us).
+constexpr SplitShapeSel lds_split_gated_shape(bool bf16, int K) { return SplitShapeSel{bf16 ? 2 : 1, K >= 31 ? 10 : 12, 4, 2}; }
 // LayerNorm-fused forward: one 2 KiB column block holds a whole row (C <= 1024 in bf16, 512 in fp32); 4 wave-columns x 8
 // bytes per lane, 2 row groups of 8 rows (16-row tiles of K + 15 staged rows), 8 compute + 8 loader waves, three tiles
 // (one computed, one having its row statistics taken by the loader waves, one in flight: 132 KiB at K = 7). With two
@@ -317,7 +329,7 @@ constexpr LdsShapeSel lds_gated_shape(bool bwd, bool bf16, bool narrow = false, 
     return LdsShapeSel{bf16, bf16 ? 2 : 1, 16, 2, 4, 4, 2};
 }
 constexpr bool lds_gated_kernel_size(int K, bool bwd) { return K == 3 || K == 5 || K == 7 || K == 9 || (!bwd && (K == 15 || K == 31)); }
-constexpr bool long_gated_kernel_size(int K) { return K == 15 || K == 31; }   // backward: sliding-window kernel, gated
+constexpr bool long_gated_kernel_size(int K) { return K == 15 || K == 31; }   // backward: role-split kernel (GATED), else sliding-window
 constexpr int default_maxt(bool bwd, int K, int vec) {
     (void)bwd; (void)K; (void)vec;
     return 256;

@@ -38,8 +38,10 @@
 namespace nplm {
 
 // FWD: the forward (y from x), which is the dx role alone on every wave, with the taps in forward order and the bias.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD = false>
+// GATED (backward only): x is z = [u | g] of shape [T, 2C] and a buffer holds a u tile and a g tile behind the dy tile.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD = false, bool GATED = false>
 struct SplitShape {
+    static_assert(!(FWD && GATED), "the gated forward forms its gate in LDS on loader waves (dwconv_lds_kernels.h)");
     static constexpr int E = BF16 ? 2 : 4;
     static constexpr int P = (K - 1) / 2;
     static constexpr int NROLE = FWD ? 1 : 2;
@@ -59,12 +61,13 @@ struct SplitShape {
     static constexpr int CB_CH = NCW * 64 * VEC;
     static constexpr int CPR = CB_BYTES / 16;              // 16-byte chunks per staged row
     static constexpr int IN_BYTES = NROWS * CB_BYTES;      // dy tile
-    static constexpr int X_BYTES = FWD ? 0 : R * CB_BYTES; // backward: x tile, no halo
-    static constexpr int BUF_BYTES = IN_BYTES + X_BYTES;
+    static constexpr int X_BYTES = FWD ? 0 : R * CB_BYTES; // backward: x tile, no halo (gated: the u tile, and as much again for g)
+    static constexpr int BUF_BYTES = IN_BYTES + X_BYTES * (GATED ? 2 : 1);
     static constexpr int LDS_BYTES = 2 * BUF_BYTES;
     static constexpr int RPL = 64 / CPR;                   // staged rows per 1 KiB load (64 lanes x 16 bytes)
     static constexpr int NLD_IN = (NROWS + RPL - 1) / RPL; // loads of a dy tile
-    static constexpr int NLD_X = FWD ? 0 : (R + RPL - 1) / RPL;   // loads of an x tile
+    static constexpr int NLD_X1 = FWD ? 0 : (R + RPL - 1) / RPL;  // loads of an x tile (gated: of the u tile, of the g tile)
+    static constexpr int NLD_X = NLD_X1 * (GATED ? 2 : 1);
     static_assert(CB_BYTES == 256 || CB_BYTES == 512 || CB_BYTES == 1024, "a staged row is 16, 32 or 64 chunks");
     static_assert(NW <= 16, "at most 1024 threads per block");
     static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers must fit in LDS");
@@ -94,12 +97,17 @@ __device__ __forceinline__ void lds_read_pinned(const char* p, RowVec<BF16, VEC>
 // with both roles' K per-channel values meeting at every join needs 170 registers where either role needs 106).
 // Both execute the same sequence of barriers.
 // Backward: in = dy, other = x, out = dx, partial = dw/db slabs. Forward: in = x, out = y, bias may be null.
-template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD, int ROLE>
+// GATED (backward): other = z = [u | g] [T, 2C], the conv ran over h = u * silu(g), out = dz [T, 2C]. The dw/db role
+// forms h of its rows as it reads them; the dx role reads u and g of an output row when its last tap is in and stores
+//     du = dh * g * sig(g),   dg = dh * u * sig(g) * (1 + g * (1 - sig(g))),   dh = the conv's input gradient.
+// Each role evaluates the sigmoid of its rows itself (once per element and role): handing it over through LDS would
+// need 8 bytes per element where u and g leave 4.
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD, int ROLE, bool GATED = false>
 __device__ __forceinline__ void split_role(const void* __restrict__ in, const void* __restrict__ other,
                                            const int32_t* __restrict__ cu, const void* __restrict__ w,
                                            const void* __restrict__ bias, void* __restrict__ out,
                                            float* __restrict__ partial, const LdsGeo& g) {
-    using SH = SplitShape<BF16, K, VEC, RW, NRG, NCW, FWD>;
+    using SH = SplitShape<BF16, K, VEC, RW, NRG, NCW, FWD, GATED>;
     constexpr int P = SH::P, E = SH::E, R = SH::R, NJ = SH::NJ, NROLE = SH::NROLE;
     using Row = RowVec<BF16, VEC>;
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
@@ -123,6 +131,8 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     const int lc0 = active ? lcol : cw - VEC;
     const int c0 = cb * SH::CB_CH + lc0;
     const int out_voff = c0 * E;
+    const int xrowb = GATED ? 2 * rowb : rowb;             // pitch of x and of the output (z and dz when gated)
+    const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;
 
     // ---- staging: direct global->LDS loads of 1 KiB (64 lanes x 16 bytes = RPL adjacent rows of the column block) ----
     // A tile is one run of 16-byte chunks, dy rows first (NLD_IN loads), then x rows (NLD_X loads); load number
@@ -133,6 +143,8 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     // row masks), and a wave that stores dx and also waits for loads is the only kind that waits for store
     // acknowledgements at the tile's barrier; the dw/db role never waits on memory.
     // (In the forward every wave is of that kind.)
+    // (Gated, where the dx role is the heavier one - the gate's derivative and two stores per output row - the dw/db role
+    // staging the tiles instead measured 779 against 738 us at T=131072, C=2048, K=31.)
     constexpr bool LOADS = ROLE == 0;
     constexpr int NLW = SH::NW / NROLE;                                         // waves that stage tiles
     constexpr int NPW = (SH::NLD_IN + SH::NLD_X + NLW - 1) / NLW;               // loads per such wave and tile
@@ -149,10 +161,11 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     char* nbuf = lds_raw;
     int lw_t = lw;              // lw, made opaque in every tile: see stage_begin
     const int v_lane = lrow * rowb + col_byte0 + lchunk * 16;
+    const int v_lane_x = lrow * xrowb + col_byte0 + lchunk * 16;
     auto stage_begin = [&](char* buf, int t0) __attribute__((always_inline)) {
         const int rb = t0 - P > 0 ? t0 - P : 0;
         rs_in = rows_rsrc(in, rb, T, row_bytes);
-        if constexpr (!FWD) rs_x = rows_rsrc(other, t0, T, row_bytes);
+        if constexpr (!FWD) rs_x = rows_rsrc(other, t0, T, x_row_bytes);
         s_in = (t0 - P - rb) * rowb;
         nbuf = buf;
         // everything a load derives from the wave's index is the same in every tile; computed once outside the tile
@@ -167,9 +180,13 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             if (lane_ok && (SH::NROWS % SH::RPL == 0 || gi * SH::RPL + lrow < SH::NROWS))
                 load_to_lds<FWD ? kLoadAuxOnceFwd : kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * rowb)), 0, once);
         } else if (gi < SH::NLD_IN + SH::NLD_X) {
-            const int i = gi - SH::NLD_IN;
+            // gated: the loads of the u tile, then those of the g tile (the second half of every z row)
+            const int i2 = gi - SH::NLD_IN;
+            const bool gpart = GATED && i2 >= SH::NLD_X1;
+            const int i = gpart ? i2 - SH::NLD_X1 : i2;
             if (lane_ok && (R % SH::RPL == 0 || i * SH::RPL + lrow < R))
-                load_to_lds<kLoadAuxOnceBwdX>(rs_x, nbuf + SH::IN_BYTES + i * 1024, v_lane + i * (SH::RPL * rowb), 0, true);
+                load_to_lds<kLoadAuxOnceBwdX>(rs_x, nbuf + SH::IN_BYTES + (gpart ? SH::X_BYTES : 0) + i * 1024,
+                                              v_lane_x + (gpart ? rowb : 0) + i * (SH::RPL * xrowb), 0, true);
         }
     };
     bool spread = false;        // the loads of the next tile are issued from inside the row schedule
@@ -231,6 +248,48 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     __syncthreads();
 
     rsrc_t ro;                  // output rows of the wave in the current tile (dx role)
+    const char* lpx_cur = lds_raw;     // x rows of the wave in the current tile: row u <-> global row tf + u (gated: u rows, g rows X_BYTES on)
+    // dx role: output row u of the wave from its finished row sum (gated: the two halves of the dz row)
+    auto emit_row = [&](int u, const float (&acc)[VEC]) __attribute__((always_inline)) {
+        if constexpr (GATED) {
+            // (pinned reads: this wave has direct loads in flight, see lds_read_pinned)
+            float uu[VEC], gg[VEC], du[VEC], dg[VEC];
+            Row ru, rg_;
+            lds_read_pinned<BF16, VEC>(lpx_cur + u * SH::CB_BYTES, ru);
+            lds_read_pinned<BF16, VEC>(lpx_cur + SH::X_BYTES + u * SH::CB_BYTES, rg_);
+            ru.to_f32(uu);
+            rg_.to_f32(gg);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+                const float sg = sigmoid_f32(gg[v]);
+                du[v] = acc[v] * (gg[v] * sg);
+                dg[v] = acc[v] * (uu[v] * sg * (1.f + gg[v] * (1.f - sg)));
+            }
+            Row ou, og;
+            ou.from_f32(du);
+            og.from_f32(dg);
+            if (active) {
+                ou.bstore(ro, out_voff, u * xrowb);
+                og.bstore(ro, out_voff + rowb, u * xrowb);
+            }
+        } else {
+            Row o;
+            o.from_f32(acc);
+            if (active) o.bstore(ro, out_voff, u * xrowb);
+        }
+    };
+    // dw role: x row u of the wave as the conv saw it (gated: h = u * silu(g))
+    auto read_x_row = [&](int u, float (&xv)[VEC]) __attribute__((always_inline)) {
+        if constexpr (GATED) {
+            float uu[VEC], gg[VEC];
+            lds_read_row<BF16, VEC>(lpx_cur + u * SH::CB_BYTES, uu);
+            lds_read_row<BF16, VEC>(lpx_cur + SH::X_BYTES + u * SH::CB_BYTES, gg);
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) xv[v] = gate_mul(uu[v], gg[v]);
+        } else {
+            lds_read_row<BF16, VEC>(lpx_cur + u * SH::CB_BYTES, xv);
+        }
+    };
     // slot of the schedule after staged row j: the next load of the tile being staged
     auto slot = [&](auto j_c) __attribute__((always_inline)) {
         constexpr int j = decltype(j_c)::value;
@@ -248,25 +307,23 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     // row j feeds output rows u = j-K+1 .. j with tap m = j - u
     auto run_rows = [&](const char* lp, auto unmasked_c, int jlo, int jhi) __attribute__((always_inline)) {
         constexpr bool UNMASKED = decltype(unmasked_c)::value;
+        // Both forms keep two rows ahead in registers. A pass over the rows of one sequence (not UNMASKED) reads every
+        // staged row all the same and skips only the arithmetic of the rows outside [jlo, jhi): a read that waits for
+        // its row right before it is used leaves the wave idle for an LDS round trip per row, and a boundary wave that
+        // runs late holds up its whole block at the tile's barrier.
         Row nxt[2];
-        if constexpr (UNMASKED) {
-            lds_read_pinned<BF16, VEC>(lp, nxt[0]);
-            lds_read_pinned<BF16, VEC>(lp + SH::CB_BYTES, nxt[1]);
-        }
+        lds_read_pinned<BF16, VEC>(lp, nxt[0]);
+        lds_read_pinned<BF16, VEC>(lp + SH::CB_BYTES, nxt[1]);
         // (a compile-time loop: as an ordinary loop its unrolled body is too large for the unroller at K = 31, and
         // the register arrays would then be indexed at run time and live in scratch memory)
         static_for<NJ>([&](auto j_c) __attribute__((always_inline)) {
             constexpr int j = decltype(j_c)::value;
+            // the scheduling barrier below keeps the compiler from hoisting all NJ reads to the top, which would not fit
+            // the 128 registers of 4 waves per SIMD
+            float gr[VEC];
+            nxt[j & 1].to_f32(gr);
+            if (j + 2 < NJ) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[j & 1]);
             if (UNMASKED || (j >= jlo && j < jhi)) {
-                float gr[VEC];
-                if constexpr (UNMASKED) {
-                    // two rows ahead in registers; the scheduling barrier below keeps the compiler from hoisting
-                    // all NJ reads to the top, which would not fit the 128 registers of 4 waves per SIMD
-                    nxt[j & 1].to_f32(gr);
-                    if (j + 2 < NJ) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[j & 1]);
-                } else {
-                    lds_read_row<BF16, VEC>(lp + j * SH::CB_BYTES, gr);
-                }
 #pragma unroll
                 for (int u = 0; u < RW; ++u) {
                     if (j - u >= 0 && j - u < K) {
@@ -280,11 +337,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                 if constexpr (UNMASKED) {
                     pin_row(j_c);
                     // output row j - (K-1) has all its taps: out it goes, long before the tile ends
-                    if constexpr (j >= K - 1) {
-                        Row o;
-                        o.from_f32(b[j - (K - 1)]);
-                        if (active) o.bstore(ro, out_voff, (j - (K - 1)) * rowb);
-                    }
+                    if constexpr (j >= K - 1) emit_row(j - (K - 1), b[j - (K - 1)]);
                 }
             }
             if constexpr (UNMASKED) slot(j_c);
@@ -363,14 +416,19 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
             const char* lpi = cur + loff;                              // taps: staged row j <-> global row tf - P + j
             const char* lpx = cur + SH::IN_BYTES + loff;               // backward x: row u <-> global row tf + u
-            ro = rows_rsrc(out, tf, T, row_bytes);
+            lpx_cur = lpx;
+            ro = rows_rsrc(out, tf, T, x_row_bytes);
             // role 0: store output rows [u0, u1) of the wave from b
             auto store_rows = [&](int u0, int u1) __attribute__((always_inline)) {
 #pragma unroll
                 for (int u = 0; u < RW; ++u) {
-                    Row o;
-                    o.from_f32(b[u]);
-                    if (u >= u0 && u < u1 && active) o.bstore(ro, out_voff, u * rowb);
+                    if constexpr (GATED) {
+                        if (u >= u0 && u < u1) emit_row(u, b[u]);
+                    } else {
+                        Row o;
+                        o.from_f32(b[u]);
+                        if (u >= u0 && u < u1 && active) o.bstore(ro, out_voff, u * rowb);
+                    }
                 }
             };
             if constexpr (ROLE == 0) {
@@ -429,6 +487,10 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                         Row r;
                         r.load(lpx + decltype(u_c)::value * SH::CB_BYTES);
                         add_sq(r);
+                        if constexpr (GATED) {      // h = u * silu(g) is finite when u and g are (up to overflow, see above)
+                            r.load(lpx + SH::X_BYTES + decltype(u_c)::value * SH::CB_BYTES);
+                            add_sq(r);
+                        }
                     });
                     exact = __builtin_amdgcn_ballot_w64(!__builtin_isfinite(chk)) != 0;
                 }
@@ -444,7 +506,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                         jlo = __builtin_amdgcn_readfirstlane(jlo < 0 ? 0 : jlo);
                         jhi = __builtin_amdgcn_readfirstlane(jhi > NJ ? NJ : jhi);
                         float xv[VEC], gc[VEC];
-                        lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, xv);
+                        read_x_row(u, xv);
                         lds_read_row<BF16, VEC>(lpi + (u + P) * SH::CB_BYTES, gc);
 #pragma unroll
                         for (int v = 0; v < VEC; ++v) c[v] += gc[v];
@@ -475,7 +537,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                         u1 = __builtin_amdgcn_readfirstlane(u1 > RW ? RW : u1);
                     }
 #pragma unroll
-                    for (int u = 0; u < RW; ++u) lds_read_row<BF16, VEC>(lpx + u * SH::CB_BYTES, b[u]);
+                    for (int u = 0; u < RW; ++u) read_x_row(u, b[u]);
                     if (!interior) {
 #pragma unroll
                         for (int u = 0; u < RW; ++u) {
@@ -536,6 +598,17 @@ dwconv_bwd_split_kernel(const void* __restrict__ x, const void* __restrict__ dy,
         split_role<BF16, K, VEC, RW, NRG, NCW, false, 0>(dy, x, cu, w, nullptr, dx, partial, g);
     else
         split_role<BF16, K, VEC, RW, NRG, NCW, false, 1>(dy, x, cu, w, nullptr, dx, partial, g);
+}
+
+// x = z = [u | g] [T, 2C], dx = dz [T, 2C]
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
+__global__ void __launch_bounds__(NCW * 2 * NRG * 64)
+dwconv_bwd_split_gated_kernel(const void* __restrict__ z, const void* __restrict__ dy, const int32_t* __restrict__ cu,
+                              const void* __restrict__ w, void* __restrict__ dz, float* __restrict__ partial, const LdsGeo g) {
+    if (SplitShape<BF16, K, VEC, RW, NRG, NCW, false, true>::role_of(wave_id()) == 0)
+        split_role<BF16, K, VEC, RW, NRG, NCW, false, 0, true>(dy, z, cu, w, nullptr, dz, partial, g);
+    else
+        split_role<BF16, K, VEC, RW, NRG, NCW, false, 1, true>(dy, z, cu, w, nullptr, dz, partial, g);
 }
 
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>

@@ -55,7 +55,9 @@ LENS_LONG = LENS_MIX + [40, 33, 31, 30, 29, 16, 15, 14, 0, 1, 1, 700]
                                        (torch.float32, torch.float32, 776), (torch.bfloat16, torch.bfloat16, 1152)])
 def test_long_gated_kernel_sizes_and_widths(K, dt, wdt, C):
     """K = 15 and 31 (the intermediate-width configuration is C = 2048, K = 31): the forward forms the gate product in
-    LDS once per staged element, the backward is the sliding-window kernel with the gate on its centre rows."""
+    LDS once per staged element; the backward is the role-split kernel with the gate in both roles (rows of at least
+    512 bytes) or the sliding-window kernel with the gate on its centre rows (C = 256 in bf16 would be; 520 takes
+    two column blocks, the second nearly empty)."""
     print(f"[case] long gated K={K} C={C} {dt} w {wdt}", flush=True)
     _check(*_case(LENS_LONG, C, K, dt, wdt, seed=K + C), f"gated K={K} C={C} {dt}")
     _check(*_case(LENS_LONG[::-1], C, K, dt, wdt, seed=K + C + 1), f"gated residual K={K} C={C} {dt}", residual=True)
@@ -72,6 +74,31 @@ def test_long_gated_is_deterministic_and_takes_the_boundary_stress_mix():
     b = npa.gated_dwconv_bwd(zd, dyd, cud, wd)
     assert all(torch.equal(p, q) for p, q in zip(a, b))
     assert torch.equal(npa.gated_dwconv_fwd(zd, cud, wd, None), npa.gated_dwconv_fwd(zd, cud, wd, None))
+
+
+@pytest.mark.parametrize("C,K,dt", [(1024, 7, torch.bfloat16), (2048, 31, torch.bfloat16), (1024, 15, torch.bfloat16),
+                                     (512, 31, torch.float32), (1152, 5, torch.bfloat16)])
+def test_nonfinite_gate_inputs_reach_only_the_taps_their_products_belong_to(C, K, dt):
+    """As for the plain conv (test_gpu_parity): h = x_proj * silu(gate) of a sequence of L rows feeds the taps with
+    |k - P| < L only, so an Inf in x_proj or a NaN in gate of one- and two-row sequences must leave the other taps of dw
+    and all of db bit for bit as they are without it; the boundary paths of the gated kernels mask by selection."""
+    lens = [40, 1, 2, 50, 1, 300, 2, 30, 7, 1, 213, 2, 64, 1, 33, 700, 2, 1]
+    P = (K - 1) // 2
+    z, cu, w, b, dy = _case(lens, C, K, dt, dt, seed=C + K)
+    cul = cu.tolist()
+    zd, cud, wd, dyd = (t.to(DEV) for t in (z, cu, w, dy))
+    _, dw0, db0 = npa.gated_dwconv_bwd(zd, dyd, cud, wd)
+    for what, L, col0, val in (("Inf in x_proj of one-row sequences", 1, 0, float("inf")),
+                               ("NaN in gate of two-row sequences", 2, C, float("nan"))):
+        z2 = z.clone()
+        for i, n in enumerate(lens):
+            if n == L:
+                z2[cul[i]:cul[i + 1], col0:col0 + C] = val
+        _, dw, db = npa.gated_dwconv_bwd(z2.to(DEV), dyd, cud, wd)
+        touched = torch.tensor([abs(k - P) <= L - 1 for k in range(K)])
+        assert bool((~torch.isfinite(dw[:, touched])).all()), f"{what}: a tap the rows feed stayed finite"
+        assert torch.equal(dw[:, ~touched], dw0[:, ~touched]), f"{what}: a tap the rows do not feed changed"
+        assert torch.equal(db, db0), f"{what}: db changed"
 
 
 def test_gated_intermediate_width_with_fp32_weights_and_residual():
