@@ -68,7 +68,8 @@ extern "C" {
 
 /* flags of the _ex entry points */
 #define NPLM_DWCONV_RESIDUAL 1u   /* fuse the residual connection: y = x + conv(x), dx = dy + conv^T(dy) */
-#define NPLM_DWCONV_GRADS_BF16 2u /* nplm_dwconv_bwd_ex / _static only: dw and db point to bf16 buffers */
+#define NPLM_DWCONV_GRADS_BF16 2u /* backward entry points with a flags argument: the parameter gradients (dw, db, and
+                                     dln_weight, dln_bias of nplm_dwconv_ln_bwd) point to bf16 buffers */
 
 #define NPLM_DWCONV_MAX_K 255
 

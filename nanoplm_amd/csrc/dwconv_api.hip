@@ -841,14 +841,16 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
                        int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
-    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    if (flags & ~(uint32_t)(NPLM_DWCONV_RESIDUAL | NPLM_DWCONV_GRADS_BF16)) return -NPLM_DWCONV_EFLAGS;
+    const int out_bf16 = (flags & NPLM_DWCONV_GRADS_BF16) ? 1 : 0;      // dw, db, dln_weight, dln_bias are bf16 buffers
     hipStream_t s = (hipStream_t)stream;
     if (!dw || !db || !dln_weight) return -NPLM_DWCONV_ENULL;
     if (T == 0) {
-        hipError_t e = fill_zero(dw, (long long)C * K, s);
-        if (e == hipSuccess) e = fill_zero(db, C, s);
-        if (e == hipSuccess) e = fill_zero(dln_weight, C, s);
-        if (e == hipSuccess) e = fill_zero(dln_bias, C, s);
+        auto zero = [&](float* p, long long n) { return out_bf16 ? fill_zero16(p, n, s) : fill_zero(p, n, s); };
+        hipError_t e = zero(dw, (long long)C * K);
+        if (e == hipSuccess) e = zero(db, C);
+        if (e == hipSuccess) e = zero(dln_weight, C);
+        if (e == hipSuccess) e = zero(dln_bias, C);
         return (int)e;
     }
     if (!x || !dy || !cu || !stats || !ln_weight || !w || !dx) return -NPLM_DWCONV_ENULL;
@@ -856,7 +858,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     const uintptr_t E = bf16 ? 2 : 4;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if (((uintptr_t)w | (uintptr_t)ln_weight | (uintptr_t)ln_bias) % WE || ((uintptr_t)cu | (uintptr_t)stats) % 4 ||
-        ((uintptr_t)dw | (uintptr_t)db | (uintptr_t)dln_weight | (uintptr_t)dln_bias) % 4 ||
+        ((uintptr_t)dw | (uintptr_t)db | (uintptr_t)dln_weight | (uintptr_t)dln_bias) % (out_bf16 ? 2 : 4) ||
         ((uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx) % E)
         return -NPLM_DWCONV_EALIGN;
     if (!ln_supported(bf16, C, K, (uintptr_t)x | (uintptr_t)dy | (uintptr_t)dx)) return -NPLM_DWCONV_EUNSUPPORTED;
@@ -870,7 +872,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     float* dn = reinterpret_cast<float*>(ws + l.conv_slabs + l.ln_slabs);
     // the conv's own residual flag stays off: the identity branch bypasses the LayerNorm and joins where dx is formed
     // (the WHOLE variant takes the flag to mean exactly that)
-    const int w_flags = kernel_w_flags(w_dtype, l.whole ? flags : 0);
+    const int w_flags = kernel_w_flags(w_dtype, l.whole ? (flags & NPLM_DWCONV_RESIDUAL) : 0);
     const ConvPtrs la{x, dy, cu, w, nullptr, l.whole ? dx : (void*)dn, part};
     const LnSide ln{stats, ln_weight, ln_bias, part_ln};
     const LdsGeo g = make_lds_geo(l.lp, T, C, S, w_flags);
@@ -902,7 +904,8 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
     // both slab sets in one launch; the LayerNorm slabs read as a conv of one tap: "dw" = d ln_weight, "db" = d ln_bias
     const int blocks_a = (int)(((long long)(K + 1) * C + 63) / 64), blocks_b = (int)((2LL * C + 63) / 64);
     hipLaunchKernelGGL(dwconv_finalize2_kernel<FIN_SPLIT>, dim3((unsigned)(blocks_a + blocks_b)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, (int)K, dw, db, blocks_a, (const float*)part_ln, 1, dln_weight, dln_bias, l.lp.nbt, (int)C);
+                       (const float*)part, (int)K, dw, db, blocks_a, (const float*)part_ln, 1, dln_weight, dln_bias, l.lp.nbt, (int)C,
+                       out_bf16);
     if (l.whole) return (int)hipGetLastError();
     const void* res = (flags & NPLM_DWCONV_RESIDUAL) ? dy : nullptr;
     const int nch = ln_row_chunks((long long)C * (long long)E);
@@ -936,18 +939,19 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
                           int32_t S, int32_t act_dtype, int32_t w_dtype, uint32_t flags, void* stream) {
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
-    if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
+    if (flags & ~(uint32_t)(NPLM_DWCONV_RESIDUAL | NPLM_DWCONV_GRADS_BF16)) return -NPLM_DWCONV_EFLAGS;
+    const int out_bf16 = (flags & NPLM_DWCONV_GRADS_BF16) ? 1 : 0;      // dw, db are bf16 buffers
     hipStream_t s = (hipStream_t)stream;
     if (!dw || !db) return -NPLM_DWCONV_ENULL;
     if (T == 0) {
-        hipError_t e = fill_zero(dw, (long long)C * K, s);
-        if (e == hipSuccess) e = fill_zero(db, C, s);
+        hipError_t e = out_bf16 ? fill_zero16(dw, (long long)C * K, s) : fill_zero(dw, (long long)C * K, s);
+        if (e == hipSuccess) e = out_bf16 ? fill_zero16(db, C, s) : fill_zero(db, C, s);
         return (int)e;
     }
     if (!z || !dy || !cu || !w || !dz) return -NPLM_DWCONV_ENULL;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
-    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % 4) return -NPLM_DWCONV_EALIGN;
+    if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % (out_bf16 ? 2 : 4)) return -NPLM_DWCONV_EALIGN;
     if (long_gated_kernel_size(K) && split_gated_eligible(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
         LdsPlan lp;
         rc = make_split_plan(false, bf16, T, C, K, nullptr, &lp, true);
@@ -962,7 +966,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, lp.nbt, C, K, dw, db, 0);
+                           (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
         return (int)hipGetLastError();
     }
     if (long_gated_bwd_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
@@ -981,7 +985,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, p.nbt, C, K, dw, db, 0);
+                           (const float*)part, p.nbt, C, K, dw, db, out_bf16);
         return (int)hipGetLastError();
     }
     if (!gated_supported(true, bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
@@ -1006,7 +1010,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     if (e != hipSuccess) return (int)e;
     const long long n_out = (long long)(K + 1) * C;
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, lp.nbt, C, K, dw, db, 0);
+                       (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
     return (int)hipGetLastError();
 }
 

@@ -552,10 +552,11 @@ __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float
 template <int SPLIT>
 __global__ void __launch_bounds__(64 * SPLIT)
 dwconv_finalize2_kernel(const float* __restrict__ pa, int Ka, float* __restrict__ dwa, float* __restrict__ dba, int blocks_a,
-                        const float* __restrict__ pb, int Kb, float* __restrict__ dwb, float* __restrict__ dbb, int nbt, int C) {
+                        const float* __restrict__ pb, int Kb, float* __restrict__ dwb, float* __restrict__ dbb, int nbt, int C,
+                        int out_bf16) {
     __shared__ float red[SPLIT][64];
-    if ((int)blockIdx.x < blocks_a) finalize_block<SPLIT>(red, (int)blockIdx.x, pa, nbt, C, Ka, dwa, dba);
-    else finalize_block<SPLIT>(red, (int)blockIdx.x - blocks_a, pb, nbt, C, Kb, dwb, dbb);
+    if ((int)blockIdx.x < blocks_a) finalize_block<SPLIT>(red, (int)blockIdx.x, pa, nbt, C, Ka, dwa, dba, out_bf16);
+    else finalize_block<SPLIT>(red, (int)blockIdx.x - blocks_a, pb, nbt, C, Kb, dwb, dbb, out_bf16);
 }
 
 // =============================================================================================

@@ -84,8 +84,9 @@ def gated_dwconv_fwd(z, cu_seqlens, weight, bias=None, *, residual: bool = False
     return y
 
 
-def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
-    """Raw backward: (dz [T, 2C] in z's dtype, dw [C, K] fp32, db [C] fp32); unsupported shapes as in the forward."""
+def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False, grads_bf16: bool = False):
+    """Raw backward: (dz [T, 2C] in z's dtype, dw [C, K] fp32, db [C] fp32); unsupported shapes as in the forward.
+    With ``grads_bf16`` dw and db come back in bf16, rounded once by the reduction kernel that forms them."""
     T, C, K, S = _check(z, cu_seqlens, weight, None)
     if tuple(dy.shape) != (T, C) or dy.dtype != z.dtype or dy.device != z.device:
         raise ValueError("dy must be [T, C] in z's dtype on z's device")
@@ -99,15 +100,17 @@ def gated_dwconv_bwd(z, dy, cu_seqlens, weight, *, residual: bool = False):
         rc = -_lib.EUNSUPPORTED
         if nbytes > 0 or T == 0:
             dz = torch.empty_like(z)
-            dw = torch.empty((C, K), dtype=torch.float32, device=z.device)
-            db = torch.empty((C,), dtype=torch.float32, device=z.device)
+            gdt = torch.bfloat16 if grads_bf16 else torch.float32
+            dw = torch.empty((C, K), dtype=gdt, device=z.device)
+            db = torch.empty((C,), dtype=gdt, device=z.device)
             ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=z.device)
             rc = lib.nplm_dwconv_gated_bwd(_ptr(z), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(weight), _ptr(dz), _ptr(dw),
                                            _ptr(db), _ptr(ws), ws.numel(), T, C, K, S, act, _DTYPES[weight.dtype],
-                                           _lib.RESIDUAL if residual else 0, dev.stream)
+                                           (_lib.RESIDUAL if residual else 0) | (_lib.GRADS_BF16 if grads_bf16 else 0),
+                                           dev.stream)
     if rc == -_lib.EUNSUPPORTED:
         uf, gs, sg, gf = _gate_terms(z)
-        dh, dw, db = varlen_dwconv_bwd((uf * gs).to(z.dtype), dy, cu_seqlens, weight, residual=residual)
+        dh, dw, db = varlen_dwconv_bwd((uf * gs).to(z.dtype), dy, cu_seqlens, weight, residual=residual, grads_bf16=grads_bf16)
         dhf = dh.float()
         dz = torch.cat((dhf * gs, dhf * uf * sg * (1.0 + gf * (1.0 - sg))), dim=-1).to(z.dtype)
         return dz, dw, db
@@ -131,7 +134,8 @@ class GatedVarlenDWConv1dFunction(torch.autograd.Function):
         z, cu_seqlens, weight = ctx.saved_tensors
         if dy.dtype != z.dtype:
             dy = dy.to(z.dtype)
-        dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=ctx.residual)
+        grads_bf16 = weight.dtype == torch.bfloat16 and ctx.bias_dtype in (None, torch.bfloat16)
+        dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=ctx.residual, grads_bf16=grads_bf16)
         return (dz if ctx.needs_input_grad[0] else None, None,
                 dw.to(weight.dtype) if ctx.needs_input_grad[2] else None,
                 db.to(ctx.bias_dtype) if (ctx.bias_dtype is not None and ctx.needs_input_grad[3]) else None, None)
@@ -165,16 +169,17 @@ def _(z, cu_seqlens, weight, bias, residual=False):
 
 @torch.library.custom_op("nanoplm_amd::gated_dwconv_bwd", mutates_args=(), device_types="cuda")
 def gated_dwconv_bwd_op(z: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, weight: torch.Tensor,
-                        residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=residual)
+                        residual: bool = False, grads_bf16: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    dz, dw, db = gated_dwconv_bwd(z, dy, cu_seqlens, weight, residual=residual, grads_bf16=grads_bf16)
     return dz, dw, db
 
 
 @gated_dwconv_bwd_op.register_fake
-def _(z, dy, cu_seqlens, weight, residual=False):
+def _(z, dy, cu_seqlens, weight, residual=False, grads_bf16=False):
     C, K = weight.shape
+    gdt = torch.bfloat16 if grads_bf16 else torch.float32
     return (torch.empty_like(z, memory_format=torch.contiguous_format),
-            z.new_empty((C, K), dtype=torch.float32), z.new_empty((C,), dtype=torch.float32))
+            z.new_empty((C, K), dtype=gdt), z.new_empty((C,), dtype=gdt))
 
 
 def _gated_setup_context(ctx, inputs, output):
@@ -188,7 +193,8 @@ def _gated_backward(ctx, dy):
     z, cu_seqlens, weight = ctx.saved_tensors
     if dy.dtype != z.dtype:
         dy = dy.to(z.dtype)
-    dz, dw, db = gated_dwconv_bwd_op(z, dy.contiguous(), cu_seqlens, weight, ctx.residual)
+    grads_bf16 = weight.dtype == torch.bfloat16 and ctx.bias_dtype in (None, torch.bfloat16)
+    dz, dw, db = gated_dwconv_bwd_op(z, dy.contiguous(), cu_seqlens, weight, ctx.residual, grads_bf16)
     return dz, None, dw.to(weight.dtype), (None if ctx.bias_dtype is None else db.to(ctx.bias_dtype)), None
 
 

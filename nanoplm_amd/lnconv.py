@@ -94,9 +94,11 @@ def ln_dwconv_fwd(x, cu_seqlens, ln_weight, ln_bias, weight, bias=None, *, eps: 
     return y, (stats if want_stats else None)
 
 
-def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, residual: bool = False):
+def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, residual: bool = False, grads_bf16: bool = False):
     """Raw backward of :func:`ln_dwconv_fwd`: ``(dx, dln_weight, dln_bias, dw, db)``; dx in x's dtype, the rest fp32
     (dln_bias None without ``ln_bias``). ``stats`` is the forward's ``[T, 2]`` (mean, rstd).
+
+    With ``grads_bf16`` the four parameter gradients come back in bf16, rounded once by the reduction kernel.
 
     Fused shapes: the conv backward normalises x as it reads it (the normalised tensor is never stored) and sums the
     LayerNorm parameter gradients beside dw and db; dx comes from the same kernel (rows of at most 4 KiB) or from one
@@ -119,16 +121,17 @@ def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, resid
     nbytes = int(lib.nplm_dwconv_ln_bwd_workspace_bytes(T, C, K, act)) if T > 0 else 0
     if nbytes > 0 or T == 0:
         dx = torch.empty_like(x)
-        dw = torch.empty((C, K), dtype=torch.float32, device=x.device)
-        db = torch.empty((C,), dtype=torch.float32, device=x.device)
-        dg = torch.empty((C,), dtype=torch.float32, device=x.device)
-        dbeta = None if ln_bias is None else torch.empty((C,), dtype=torch.float32, device=x.device)
+        gdt = torch.bfloat16 if grads_bf16 else torch.float32
+        dw = torch.empty((C, K), dtype=gdt, device=x.device)
+        db = torch.empty((C,), dtype=gdt, device=x.device)
+        dg = torch.empty((C,), dtype=gdt, device=x.device)
+        dbeta = None if ln_bias is None else torch.empty((C,), dtype=gdt, device=x.device)
         with _launch_on(x) as dev:
             workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
             rc = lib.nplm_dwconv_ln_bwd(_ptr(x), _ptr(dy), _ptr(cu_seqlens.contiguous()), _ptr(stats), _ptr(lnw), _ptr(lnb),
                                         _ptr(weight), _ptr(dx), _ptr(dw), _ptr(db), _ptr(dg), _ptr(dbeta), _ptr(workspace),
                                         workspace.numel(), T, C, K, S, act, _DTYPES[wdt],
-                                        _lib.RESIDUAL if residual else 0, dev.stream)
+                                        (_lib.RESIDUAL if residual else 0) | (_lib.GRADS_BF16 if grads_bf16 else 0), dev.stream)
         if rc != -_lib.EUNSUPPORTED:
             _lib.check(rc, "nplm_dwconv_ln_bwd")
             return dx, dg, dbeta, dw, db
@@ -144,7 +147,16 @@ def ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, *, resid
                                                               [True, True, lnb is not None])
     if residual:
         dx = dx + dyf
+    if grads_bf16:
+        dg, dw, db = dg.bfloat16(), dw.bfloat16(), db.bfloat16()
+        dbeta = None if dbeta is None else dbeta.bfloat16()
     return dx.to(x.dtype), dg, (dbeta if lnb is not None else None), dw, db
+
+
+def _all_bf16(ln_weight, ln_bias, weight, bias_dtype) -> bool:
+    """Every parameter is bf16: their gradients can come in bf16 straight from the reduction kernel."""
+    return (weight.dtype == torch.bfloat16 and ln_weight.dtype == torch.bfloat16 and bias_dtype in (None, torch.bfloat16)
+            and (ln_bias is None or ln_bias.dtype == torch.bfloat16))
 
 
 class LnVarlenDWConv1dFunction(torch.autograd.Function):
@@ -165,7 +177,8 @@ class LnVarlenDWConv1dFunction(torch.autograd.Function):
         x, cu, ln_weight, ln_bias, weight, stats = ctx.saved_tensors
         if dy.dtype != x.dtype:
             dy = dy.to(x.dtype)
-        dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu, stats, ln_weight, ln_bias, weight, residual=ctx.residual)
+        dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu, stats, ln_weight, ln_bias, weight, residual=ctx.residual,
+                                              grads_bf16=_all_bf16(ln_weight, ln_bias, weight, ctx.bias_dtype))
         return (dx, None, dg.to(ln_weight.dtype), None if ln_bias is None else dbeta.to(ln_bias.dtype),
                 dw.to(weight.dtype), db.to(ctx.bias_dtype) if ctx.has_bias else None, None, None)
 
@@ -195,19 +208,20 @@ def _(x, cu_seqlens, ln_weight, ln_bias, weight, bias, eps=1e-5, residual=False)
 
 @torch.library.custom_op("nanoplm_amd::ln_dwconv_bwd", mutates_args=(), device_types="cuda")
 def ln_dwconv_bwd_op(x: torch.Tensor, dy: torch.Tensor, cu_seqlens: torch.Tensor, stats: torch.Tensor, ln_weight: torch.Tensor,
-                     ln_bias: Optional[torch.Tensor], weight: torch.Tensor,
-                     residual: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+                     ln_bias: Optional[torch.Tensor], weight: torch.Tensor, residual: bool = False,
+                     grads_bf16: bool = False) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dx, dln_weight, dln_bias, dw, db); dln_bias is zeros [C] without ``ln_bias`` (an op returns tensors only)."""
-    dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=residual)
+    dx, dg, dbeta, dw, db = ln_dwconv_bwd(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=residual,
+                                          grads_bf16=grads_bf16)
     if dbeta is None:
         dbeta = torch.zeros_like(dg)
     return dx, dg, dbeta, dw, db
 
 
 @ln_dwconv_bwd_op.register_fake
-def _(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=False):
+def _(x, dy, cu_seqlens, stats, ln_weight, ln_bias, weight, residual=False, grads_bf16=False):
     C, K = weight.shape
-    f = lambda *shape: x.new_empty(shape, dtype=torch.float32)
+    f = lambda *shape: x.new_empty(shape, dtype=torch.bfloat16 if grads_bf16 else torch.float32)
     return torch.empty_like(x, memory_format=torch.contiguous_format), f(C), f(C), f(C, K), f(C)
 
 
@@ -225,7 +239,8 @@ def _ln_backward(ctx, dy, _dstats):
         dy = torch.zeros_like(x)
     if dy.dtype != x.dtype:
         dy = dy.to(x.dtype)
-    dx, dg, dbeta, dw, db = ln_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, stats, ln_weight, ln_bias, weight, ctx.residual)
+    dx, dg, dbeta, dw, db = ln_dwconv_bwd_op(x, dy.contiguous(), cu_seqlens, stats, ln_weight, ln_bias, weight, ctx.residual,
+                                             _all_bf16(ln_weight, ln_bias, weight, ctx.bias_dtype))
     return (dx, None, dg.to(ln_weight.dtype), None if ln_bias is None else dbeta.to(ln_bias.dtype), dw.to(weight.dtype),
             None if ctx.bias_dtype is None else db.to(ctx.bias_dtype), None, None)
 

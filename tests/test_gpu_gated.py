@@ -101,6 +101,17 @@ def test_nonfinite_gate_inputs_reach_only_the_taps_their_products_belong_to(C, K
         assert torch.equal(db, db0), f"{what}: db changed"
 
 
+@pytest.mark.parametrize("C,K", [(1024, 7), (2048, 31), (100, 7)])
+def test_gated_parameter_gradients_straight_in_bf16(C, K):
+    """NPLM_DWCONV_GRADS_BF16 on the gated backward (fused kernels and the composed fallback): the cast of the fp32 result."""
+    z, cu, w, b, dy = _case(LENS_MIX, C, K, torch.bfloat16, torch.bfloat16, seed=C + K)
+    zd, cud, wd, dyd = (t.to(DEV) for t in (z, cu, w, dy))
+    dz, dw, db = npa.gated_dwconv_bwd(zd, dyd, cud, wd)
+    dz2, dw2, db2 = npa.gated_dwconv_bwd(zd, dyd, cud, wd, grads_bf16=True)
+    assert dw2.dtype == torch.bfloat16 and db2.dtype == torch.bfloat16
+    assert torch.equal(dz, dz2) and torch.equal(dw.bfloat16(), dw2) and torch.equal(db.bfloat16(), db2)
+
+
 def test_gated_intermediate_width_with_fp32_weights_and_residual():
     _check(*_case(LENS_MIX, 2048, 7, torch.bfloat16, torch.float32, seed=4), "gated C=2048 bf16/fp32")
     _check(*_case(LENS_MIX, 1024, 7, torch.bfloat16, torch.bfloat16, seed=6), "gated residual", residual=True)

@@ -200,6 +200,25 @@ def test_fp32_layernorm_parameters_beside_bf16_taps_are_not_rounded(dt, C):
     _check_bwd(x, cu, gam, bet, w, b, dy, f"mixed ln dtypes bwd C={C} {dt}", residual=True)
 
 
+@pytest.mark.parametrize("dt,C", [(torch.bfloat16, 1024), (torch.bfloat16, 2048), (torch.bfloat16, 3072), (torch.bfloat16, 4104)])
+def test_layernorm_parameter_gradients_straight_in_bf16(dt, C):
+    """NPLM_DWCONV_GRADS_BF16 on the LayerNorm-fused backward (one-kernel, two-kernel and composed paths): all four
+    parameter gradients equal the cast of the fp32 results; through autograd bf16 parameters get bf16 gradients."""
+    x, cu, gam, bet, w, b, dy = _case(LENS_MIX, C, 7, dt, torch.bfloat16, seed=C + 9)
+    xd, cud, gd, hd, wd, dyd = (t.to(DEV) for t in (x, cu, gam, bet, w, dy))
+    _, stats = npa.ln_dwconv_fwd(xd, cud, gd, hd, wd, None, residual=True)
+    ref = npa.ln_dwconv_bwd(xd, dyd, cud, stats, gd, hd, wd, residual=True)
+    got = npa.ln_dwconv_bwd(xd, dyd, cud, stats, gd, hd, wd, residual=True, grads_bf16=True)
+    assert torch.equal(ref[0], got[0])
+    for a, g in zip(ref[1:], got[1:]):
+        assert g.dtype == torch.bfloat16 and torch.equal(a.bfloat16(), g)
+    xr = xd.clone().requires_grad_(True)
+    params = [t.clone().requires_grad_(True) for t in (gd, hd, wd, b.to(DEV))]
+    npa.ln_varlen_dwconv(xr, cud, *params, residual=True).backward(dyd)
+    assert all(p.grad.dtype == torch.bfloat16 for p in params)
+    assert torch.equal(params[2].grad, got[3]) and torch.equal(params[0].grad, got[1])
+
+
 def test_fused_layernorm_backward_is_deterministic_and_takes_the_boundary_stress_mix():
     wl = make_workload(5, T=20011, C=1024, with_dy=True)        # lengths of 1..8 mixed with 400..512, odd T
     g = torch.Generator().manual_seed(6)
