@@ -810,6 +810,10 @@ int ln_bwd_layout(bool bf16, long long T, int C, int K, LnBwdLayout* out) {
         l.lp.ntiles = ceil_div(T, l.lp.R);
         l.lp.nbt = l.lp.ntiles < kNumCU ? l.lp.ntiles : kNumCU;
         l.lp.xcd_group = (l.lp.nbt % (kNumXCD * 8) == 0) ? 8 : 0;
+        // rows of 2 to 4 KiB: a tile is 5 to 10 rows behind K-1 halo rows of dy, and a neighbour on another XCD means reading
+        // those from HBM again (fp32 C=1024, K=7: 6-row tiles, HBM-side reads 1.066 of x + dy with 8 consecutive tiles per
+        // XCD); 32 consecutive tiles per XCD, as in the forward of these rows
+        if (l.whole4k && l.lp.nbt % (kNumXCD * 32) == 0) l.lp.xcd_group = 32;
         l.lp.rot_step = l.lp.nbt > 2 ? (int)((long long)l.lp.nbt * 618 / 1000) | 1 : 0;
         if (l.lp.rot_step >= l.lp.nbt) l.lp.rot_step = l.lp.nbt - 1;
     } else {
