@@ -49,19 +49,24 @@ VALU_PEAK_TFLOPS = 157.3  # MI355X fp32 vector ALU (256 CUs x 4 SIMDs x 32 FMA l
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this benchmark and
 # scaled by what the same counters read for nplm_dwconv_debug_copy of known size (see
 # profiles/bench_cfg3_hbm_traffic.md and profiles/bench_cfg2_cfg4_cfg5_hbm_traffic.md): keyed by
-# (workload name, kernel). Counters cannot be read from inside this process, so a workload or variant
-# without an entry (configuration 1, --gated, --residual) reports traffic = null and says why.
+# (workload name, kernel[, variant]). Counters cannot be read from inside this process, so a workload or variant
+# without an entry (configuration 1, --residual, other widths) reports traffic = null and says why.
 MEASURED_TRAFFIC = {
-    ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136282529,                       # 1.015 x algorithmic
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544046769,                   # 1.013 x
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816835497,                  # 1.014 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1076725503,       # 1.003 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619746803,      # 1.006 x
-    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272216838,    # 1.014 x
-    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410635307,   # 1.020 x
-    # --ln (profiles/bench_cfg3_layernorm_fused_sq_hbm_counters.md); the backward figure is the fused kernel's alone
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551598297,             # 1.025 x
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830254796,            # 1.031 x
+    ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136254011,                       # 1.015 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544038670,                   # 1.013 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816855087,                  # 1.014 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1075063627,       # 1.001 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619794930,      # 1.005 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272191889,    # 1.014 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410655634,   # 1.020 x
+    # --gated --config 4 (profiles/bench_cfg4_gated_hbm_traffic.md)
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1610935816,    # 1.000 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693532724,   # 1.003 x
+    # --ln and --fp32 --ln (profiles/bench_cfg3_layernorm_fused_hbm_traffic.md); the backward figure is the fused kernel's alone
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551589166,             # 1.027 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830226314,            # 1.031 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "forward", "ln"): 1091916066,            # 1.017 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "backward", "ln"): 1641601215,           # 1.019 x
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
@@ -494,7 +499,8 @@ def main():
         flops = wl.algorithmic_flops("fwd" if kernel == "forward" else "bwd")
         tflops = flops / med / 1e6
         traffic = (MEASURED_TRAFFIC.get((wl.name, kernel, "ln")) if args.ln else
-                   None if (args.gated or args.residual) else MEASURED_TRAFFIC.get((wl.name, kernel)))
+                   MEASURED_TRAFFIC.get((wl.name, kernel, "gated")) if args.gated else
+                   None if args.residual else MEASURED_TRAFFIC.get((wl.name, kernel)))
         hbm = {"achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
                "algorithmic_bytes": nbytes, "us_at_peak": nbytes / HBM_PEAK_GBPS / 1e3}
         valu = {"achieved": tflops, "peak": VALU_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / VALU_PEAK_TFLOPS,
