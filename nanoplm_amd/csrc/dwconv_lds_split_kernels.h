@@ -351,6 +351,11 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     // single pass over all rows.
     auto run_rows_chunked = [&](const char* lp, int jlo, int jhi) __attribute__((always_inline)) {
         constexpr int CH = 12, NCH = (NJ + CH - 1) / CH;
+        // bit j: staged row j belongs to the pass (one scalar bit test per row, where two compares against the bounds
+        // and their conjunction took 5 scalar instructions)
+        static_assert(NJ < 64, "one mask bit per staged row");
+        const int lo_ = jlo < 0 ? 0 : jlo, hi_ = jhi > NJ ? NJ : jhi;
+        const uint64_t inmask = hi_ > lo_ ? (((1ull << hi_) - 1ull) & ~((1ull << lo_) - 1ull)) : 0ull;
         static_for<NCH>([&](auto ch_c) __attribute__((always_inline)) {
             constexpr int j0 = decltype(ch_c)::value * CH;
             constexpr int j1 = j0 + CH < NJ ? j0 + CH : NJ;
@@ -360,7 +365,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                 if (j0 + 1 < j1) lds_read_pinned<BF16, VEC>(lp + (j0 + 1) * SH::CB_BYTES, nxt[1]);
                 static_for<j1 - j0>([&](auto jj_c) __attribute__((always_inline)) {
                     constexpr int j = j0 + decltype(jj_c)::value;
-                    const bool in = j >= jlo && j < jhi;
+                    const bool in = (inmask >> j) & 1ull;
                     float gr[VEC];
                     if constexpr (BF16 && VEC == 2) {
                         // the row mask rides on the bf16 -> fp32 conversion: the high half by an AND, the low half by a
