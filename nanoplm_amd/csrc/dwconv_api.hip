@@ -285,7 +285,7 @@ int make_split_plan(bool fwd, bool bf16, long long T, int C, int K, const nplm_d
     nplm_dwconv_tuning z{};
     if (!tune) tune = &z;
     const int E = bf16 ? 2 : 4;
-    const SplitShapeSel sh = gated ? lds_split_gated_shape(bf16, K) : lds_split_shape(fwd, bf16, K);
+    const SplitShapeSel sh = !gated ? lds_split_shape(fwd, bf16, K) : fwd ? lds_split_gated_fwd_shape(bf16, K) : lds_split_gated_shape(bf16, K);
     const long long cb_bytes = (long long)sh.ncw * 64 * sh.vec * E;
     const long long row_bytes = (long long)C * E;
     p.R = sh.rw * sh.nrg;
@@ -695,6 +695,15 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
     if (!gated_supported(false, bf16, T, C, K, (uintptr_t)z | (uintptr_t)y)) return -NPLM_DWCONV_EUNSUPPORTED;
     LdsPlan lp;
+    if (long_gated_kernel_size(K) && split_gated_eligible(bf16, T, C, K, (uintptr_t)z | (uintptr_t)y)) {
+        rc = make_split_plan(true, bf16, T, C, K, nullptr, &lp, true);
+        if (rc) return rc;
+        const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+        const dim3 grid(lp.ncb * lp.nbt);
+        return (int)(K == 31 ? launch_fwd_split_gated_k31(bf16, la, lg, grid, (hipStream_t)stream)
+                             : launch_fwd_split_gated_k15(bf16, la, lg, grid, (hipStream_t)stream));
+    }
     rc = make_lds_plan(false, bf16, T, C, K, nullptr, &lp, true);
     if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
     const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};

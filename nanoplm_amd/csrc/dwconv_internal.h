@@ -111,13 +111,16 @@ hipError_t launch_bwd_gated_k15(bool bf16, int unroll, int maxt, const ConvPtrs&
                                 size_t shmem, hipStream_t s);
 hipError_t launch_bwd_gated_k31(bool bf16, int unroll, int maxt, const ConvPtrs& p, const Geo& g, dim3 grid, dim3 block,
                                 size_t shmem, hipStream_t s);
-// and LDS-staged forward with the gate formed in LDS by the loader waves
+// and LDS-staged forward with the gate formed in LDS by the loader waves (rows the role-split forward does not take)
 hipError_t launch_fwd_lds_gated_k15(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_lds_gated_k31(bool bf16, bool narrow, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 // role-split LDS kernels at K = 31 and 15 (fixed shape per dtype, see lds_split_shape())
 hipError_t launch_bwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_fwd_split_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_bwd_split_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+// gated role-split forward (z = [u | g] in, y out), see lds_split_gated_fwd_shape()
+hipError_t launch_fwd_split_gated_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
+hipError_t launch_fwd_split_gated_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 // gated role-split backward (z = [u | g] in, dz out), see lds_split_gated_shape()
 hipError_t launch_bwd_split_gated_k31(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
 hipError_t launch_bwd_split_gated_k15(bool bf16, const ConvPtrs& p, const LdsGeo& g, dim3 grid, hipStream_t s);
@@ -252,6 +255,16 @@ constexpr SplitShapeSel lds_split_shape(bool fwd, bool bf16, int K) {
 // length does not. Both roles evaluate the gate's sigmoid (two quarter-rate instructions per element and role),
 // which is what the kernel costs over the plain one (510 us).
 constexpr SplitShapeSel lds_split_gated_shape(bool bf16, int K) { return SplitShapeSel{bf16 ? 2 : 1, K >= 31 ? 10 : 12, 4, 2}; }
+// Gated role-split forward (K = 31, 15): a buffer holds a u tile and a g tile of R + K-1 rows each, which the waves turn
+// into one fp32 h tile in place before the row schedules run. 256-byte column blocks (one wave-column) with 16 row
+// groups of 8 rows: two buffers of 2 x 158 rows x 256 bytes = 158 KiB at K = 31. Measured at T=131072, C=2048, bf16
+// against the LDS-staged forward with 8 loader waves that gate 32-row tiles (log-normal mix / one long sequence):
+// K = 31 441 / 397 against 501 / 495 us, K = 15 372 / 340 against 420 / 419 us; y is the same bit for bit. At K = 15
+// 9 rows per wave (144-row tiles) or 512-byte column blocks with 8 row groups measure the same (377-390 / 356-359 us).
+constexpr SplitShapeSel lds_split_gated_fwd_shape(bool bf16, int K) {
+    (void)K;
+    return SplitShapeSel{bf16 ? 2 : 1, 8, 16, 1};
+}
 // LayerNorm-fused forward: one 2 KiB column block holds a whole row (C <= 1024 in bf16, 512 in fp32); 4 wave-columns x 8
 // bytes per lane, 2 row groups of 8 rows (16-row tiles of K + 15 staged rows), 8 compute + 8 loader waves, three tiles
 // (one computed, one having its row statistics taken by the loader waves, one in flight: 132 KiB at K = 7). With two

@@ -38,10 +38,13 @@
 namespace nplm {
 
 // FWD: the forward (y from x), which is the dx role alone on every wave, with the taps in forward order and the bias.
-// GATED (backward only): x is z = [u | g] of shape [T, 2C] and a buffer holds a u tile and a g tile behind the dy tile.
+// GATED, backward: x is z = [u | g] of shape [T, 2C] and a buffer holds a u tile and a g tile behind the dy tile.
+// FWD && GATED: x is z = [u | g] as well; a buffer holds a u tile and a g tile, both with their halo rows, which the waves
+// turn into one fp32 h = u * silu(g) tile in place before the row schedules run (see gate_tile in split_role).
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW, bool FWD = false, bool GATED = false>
 struct SplitShape {
-    static_assert(!(FWD && GATED), "the gated forward forms its gate in LDS on loader waves (dwconv_lds_kernels.h)");
+    static constexpr bool GF = FWD && GATED;
+    static_assert(!GF || (BF16 ? VEC == 2 : VEC == 1), "gated forward: a lane's slice of a row is 4 bytes of u and 4 of g");
     static constexpr int E = BF16 ? 2 : 4;
     static constexpr int P = (K - 1) / 2;
     static constexpr int NROLE = FWD ? 1 : 2;
@@ -62,12 +65,13 @@ struct SplitShape {
     static constexpr int CPR = CB_BYTES / 16;              // 16-byte chunks per staged row
     static constexpr int IN_BYTES = NROWS * CB_BYTES;      // dy tile
     static constexpr int X_BYTES = FWD ? 0 : R * CB_BYTES; // backward: x tile, no halo (gated: the u tile, and as much again for g)
-    static constexpr int BUF_BYTES = IN_BYTES + X_BYTES * (GATED ? 2 : 1);
+    static constexpr int BUF_BYTES = GF ? 2 * IN_BYTES : IN_BYTES + X_BYTES * (GATED ? 2 : 1);
     static constexpr int LDS_BYTES = 2 * BUF_BYTES;
     static constexpr int RPL = 64 / CPR;                   // staged rows per 1 KiB load (64 lanes x 16 bytes)
     static constexpr int NLD_IN = (NROWS + RPL - 1) / RPL; // loads of a dy tile
     static constexpr int NLD_X1 = FWD ? 0 : (R + RPL - 1) / RPL;  // loads of an x tile (gated: of the u tile, of the g tile)
-    static constexpr int NLD_X = NLD_X1 * (GATED ? 2 : 1);
+    static constexpr int NLD_X = GF ? NLD_IN : NLD_X1 * (GATED ? 2 : 1);  // gated forward: the g tile, like the u tile
+    static constexpr int ROW_UNITS = NROWS * NCW;          // gated forward: (staged row, wave-column) pairs to gate
     static_assert(CB_BYTES == 256 || CB_BYTES == 512 || CB_BYTES == 1024, "a staged row is 16, 32 or 64 chunks");
     static_assert(NW <= 16, "at most 1024 threads per block");
     static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers must fit in LDS");
@@ -83,6 +87,10 @@ template <bool BF16, int VEC>
 __device__ __forceinline__ void lds_read_pinned(const char* p, RowVec<BF16, VEC>& r) {
     if constexpr (RowVec<BF16, VEC>::BYTES == 2) {
         r.h = *(const volatile __attribute__((address_space(3))) uint16_t*)p;
+    } else if constexpr (RowVec<BF16, VEC>::BYTES == 8) {
+        // one 8-byte access: as two dword reads the lanes' 8-byte stride puts them two to a bank in each
+        const u32x2 t = *(const volatile __attribute__((address_space(3))) u32x2*)p;
+        __builtin_memcpy(&r, &t, sizeof(t));
     } else {
         constexpr int NDW = RowVec<BF16, VEC>::BYTES / 4;
         uint32_t t[NDW];
@@ -110,6 +118,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     using SH = SplitShape<BF16, K, VEC, RW, NRG, NCW, FWD, GATED>;
     constexpr int P = SH::P, E = SH::E, R = SH::R, NJ = SH::NJ, NROLE = SH::NROLE;
     using Row = RowVec<BF16, VEC>;
+    using InRow = RowVec<BF16 && !(FWD && GATED), VEC>;              // a lane's slice of a staged row as the schedules read it
     extern __shared__ __attribute__((aligned(16))) char lds_raw[];   // 2 x BUF_BYTES
 
     const int lane = (int)(threadIdx.x & 63);
@@ -131,8 +140,12 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     const int lc0 = active ? lcol : cw - VEC;
     const int c0 = cb * SH::CB_CH + lc0;
     const int out_voff = c0 * E;
-    const int xrowb = GATED ? 2 * rowb : rowb;             // pitch of x and of the output (z and dz when gated)
-    const size_t x_row_bytes = GATED ? 2 * row_bytes : row_bytes;
+    constexpr bool GF = FWD && GATED;                      // gated forward: in = z [T, 2C], out = y [T, C]
+    constexpr bool GB = GATED && !FWD;                     // gated backward: other = z, out = dz, both [T, 2C]
+    const int xrowb = GB ? 2 * rowb : rowb;                // pitch of x and of the output (z and dz in the gated backward)
+    const size_t x_row_bytes = GB ? 2 * row_bytes : row_bytes;
+    const int in_rowb = GF ? 2 * rowb : rowb;              // pitch of the staged input with halo (z in the gated forward)
+    const size_t in_row_bytes = GF ? 2 * row_bytes : row_bytes;
 
     // ---- staging: direct global->LDS loads of 1 KiB (64 lanes x 16 bytes = RPL adjacent rows of the column block) ----
     // A tile is one run of 16-byte chunks, dy rows first (NLD_IN loads), then x rows (NLD_X loads); load number
@@ -160,13 +173,13 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     int s_in = 0;               // byte offset of its first dy row from the descriptor's first row (negative in tile 0)
     char* nbuf = lds_raw;
     int lw_t = lw;              // lw, made opaque in every tile: see stage_begin
-    const int v_lane = lrow * rowb + col_byte0 + lchunk * 16;
+    const int v_lane = lrow * in_rowb + col_byte0 + lchunk * 16;
     const int v_lane_x = lrow * xrowb + col_byte0 + lchunk * 16;
     auto stage_begin = [&](char* buf, int t0) __attribute__((always_inline)) {
         const int rb = t0 - P > 0 ? t0 - P : 0;
-        rs_in = rows_rsrc(in, rb, T, row_bytes);
+        rs_in = rows_rsrc(in, rb, T, in_row_bytes);
         if constexpr (!FWD) rs_x = rows_rsrc(other, t0, T, x_row_bytes);
-        s_in = (t0 - P - rb) * rowb;
+        s_in = (t0 - P - rb) * in_rowb;
         nbuf = buf;
         // everything a load derives from the wave's index is the same in every tile; computed once outside the tile
         // loop it would occupy some 50 scalar registers (NPW loads x flags and offsets) and push others into spills
@@ -178,11 +191,17 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         if (gi < SH::NLD_IN) {
             const bool once = gi * SH::RPL >= 2 * P && gi * SH::RPL + SH::RPL <= SH::NROWS - 2 * P;   // no other tile stages it
             if (lane_ok && (SH::NROWS % SH::RPL == 0 || gi * SH::RPL + lrow < SH::NROWS))
-                load_to_lds<FWD ? kLoadAuxOnceFwd : kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * rowb)), 0, once);
-        } else if (gi < SH::NLD_IN + SH::NLD_X) {
+                load_to_lds<FWD ? kLoadAuxOnceFwd : kLoadAuxOnceBwd>(rs_in, nbuf + gi * 1024, v_lane + (s_in + gi * (SH::RPL * in_rowb)), 0, once);
+        } else if (GF && gi < 2 * SH::NLD_IN) {
+            // gated forward: the g tile (the second half of every z row) behind the u tile, the same rows
+            const int i = gi - SH::NLD_IN;
+            const bool once = i * SH::RPL >= 2 * P && i * SH::RPL + SH::RPL <= SH::NROWS - 2 * P;
+            if (lane_ok && (SH::NROWS % SH::RPL == 0 || i * SH::RPL + lrow < SH::NROWS))
+                load_to_lds<kLoadAuxOnceFwd>(rs_in, nbuf + SH::IN_BYTES + i * 1024, v_lane + rowb + (s_in + i * (SH::RPL * in_rowb)), 0, once);
+        } else if (!GF && gi < SH::NLD_IN + SH::NLD_X) {
             // gated: the loads of the u tile, then those of the g tile (the second half of every z row)
             const int i2 = gi - SH::NLD_IN;
-            const bool gpart = GATED && i2 >= SH::NLD_X1;
+            const bool gpart = GB && i2 >= SH::NLD_X1;
             const int i = gpart ? i2 - SH::NLD_X1 : i2;
             if (lane_ok && (R % SH::RPL == 0 || i * SH::RPL + lrow < R))
                 load_to_lds<kLoadAuxOnceBwdX>(rs_x, nbuf + SH::IN_BYTES + (gpart ? SH::X_BYTES : 0) + i * 1024,
@@ -251,7 +270,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     const char* lpx_cur = lds_raw;     // x rows of the wave in the current tile: row u <-> global row tf + u (gated: u rows, g rows X_BYTES on)
     // dx role: output row u of the wave from its finished row sum (gated: the two halves of the dz row)
     auto emit_row = [&](int u, const float (&acc)[VEC]) __attribute__((always_inline)) {
-        if constexpr (GATED) {
+        if constexpr (GB) {
             // (pinned reads: this wave has direct loads in flight, see lds_read_pinned)
             float uu[VEC], gg[VEC], du[VEC], dg[VEC];
             Row ru, rg_;
@@ -280,7 +299,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     };
     // dw role: x row u of the wave as the conv saw it (gated: h = u * silu(g))
     auto read_x_row = [&](int u, float (&xv)[VEC]) __attribute__((always_inline)) {
-        if constexpr (GATED) {
+        if constexpr (GB) {
             float uu[VEC], gg[VEC];
             lds_read_row<BF16, VEC>(lpx_cur + u * SH::CB_BYTES, uu);
             lds_read_row<BF16, VEC>(lpx_cur + SH::X_BYTES + u * SH::CB_BYTES, gg);
@@ -311,9 +330,9 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         // staged row all the same and skips only the arithmetic of the rows outside [jlo, jhi): a read that waits for
         // its row right before it is used leaves the wave idle for an LDS round trip per row, and a boundary wave that
         // runs late holds up its whole block at the tile's barrier.
-        Row nxt[2];
-        lds_read_pinned<BF16, VEC>(lp, nxt[0]);
-        lds_read_pinned<BF16, VEC>(lp + SH::CB_BYTES, nxt[1]);
+        InRow nxt[2];
+        lds_read_pinned(lp, nxt[0]);
+        lds_read_pinned(lp + SH::CB_BYTES, nxt[1]);
         // (a compile-time loop: as an ordinary loop its unrolled body is too large for the unroller at K = 31, and
         // the register arrays would then be indexed at run time and live in scratch memory)
         static_for<NJ>([&](auto j_c) __attribute__((always_inline)) {
@@ -322,7 +341,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             // the 128 registers of 4 waves per SIMD
             float gr[VEC];
             nxt[j & 1].to_f32(gr);
-            if (j + 2 < NJ) lds_read_pinned<BF16, VEC>(lp + (j + 2) * SH::CB_BYTES, nxt[j & 1]);
+            if (j + 2 < NJ) lds_read_pinned(lp + (j + 2) * SH::CB_BYTES, nxt[j & 1]);
             if (UNMASKED || (j >= jlo && j < jhi)) {
 #pragma unroll
                 for (int u = 0; u < RW; ++u) {
@@ -399,6 +418,31 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         });
     };
 
+    // Gated forward: the u and g rows of a landed tile become one fp32 h = u * silu(g) tile, once per staged element
+    // (a gate evaluated as the schedules read their rows would be evaluated NJ / RW times per element). A unit of work
+    // is one wave-column of one staged row, dealt round-robin to the waves: a lane takes its 4 bytes of u and of g
+    // (two adjacent channels in bf16, one in fp32) and the wave leaves the fp32 values of the wave-column's first 64
+    // channels in the unit's 256 bytes of the u tile and the rest in its 256 bytes of the g tile (fp32 activations: all
+    // in the u tile), which is where the schedules' lanes read their slices. All reads of a unit are one instruction
+    // of the wave and precede its writes, so the unit is turned in place. Volatile address-space-3 accesses: the waves
+    // have stores of the previous tile in flight, and before an ordinary LDS access the compiler would wait for them.
+    auto gate_tile = [&](char* buf) __attribute__((always_inline)) {
+        typedef volatile __attribute__((address_space(3))) uint32_t lds_u32;
+        for (int unit = wv; unit < SH::ROW_UNITS; unit += SH::NW) {
+            char* pu = buf + (unit / NCW) * SH::CB_BYTES + (unit % NCW) * 256;
+            char* pg = pu + SH::IN_BYTES;
+            const uint32_t ru = *(lds_u32*)(pu + lane * 4), rg_ = *(lds_u32*)(pg + lane * 4);
+            if constexpr (BF16) {
+                const u32x2 h = {__float_as_uint(gate_mul(bf16_lo(ru), bf16_lo(rg_))), __float_as_uint(gate_mul(bf16_hi(ru), bf16_hi(rg_)))};
+                *(volatile __attribute__((address_space(3))) u32x2*)((lane < 32 ? pu : pg) + (lane & 31) * 8) = h;
+            } else {
+                *(lds_u32*)(pu + lane * 4) = __float_as_uint(gate_mul(__uint_as_float(ru), __uint_as_float(rg_)));
+            }
+        }
+    };
+    // where a lane's slice of staged row 0 of the wave-column lies in a tile
+    const int lane_off = !GF ? lc0 * E : wc * 256 + (BF16 ? (lane < 32 ? 0 : SH::IN_BYTES) + (lane & 31) * 8 : lane * 4);
+
     int q = tb;
     for (int it = 0; it < ntl; ++it) {
         const int t0 = lds_tile_row0(g, it, q, R);
@@ -406,6 +450,10 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         char* cur = lds_raw + (it & 1) * SH::BUF_BYTES;
         const int rn = it + 1 < ntl ? lds_tile_row0(g, it + 1, qn, R) : T;
         const int tf = t0 + rg * RW;
+        if constexpr (GF) {
+            if (t0 < T) gate_tile(cur);
+            lds_barrier();                          // every wave's share of h is written
+        }
         __builtin_amdgcn_s_setprio(3);
         if constexpr (LOADS) {
             // an interior wave runs every row of its schedule exactly once: its loads go into the schedule's slots
@@ -418,7 +466,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             }
         }
         if (tf < T) {
-            const int loff = (rg * RW) * SH::CB_BYTES + lc0 * E;
+            const int loff = (rg * RW) * SH::CB_BYTES + lane_off;
             const char* lpi = cur + loff;                              // taps: staged row j <-> global row tf - P + j
             const char* lpx = cur + SH::IN_BYTES + loff;               // backward x: row u <-> global row tf + u
             lpx_cur = lpx;
@@ -427,7 +475,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
             auto store_rows = [&](int u0, int u1) __attribute__((always_inline)) {
 #pragma unroll
                 for (int u = 0; u < RW; ++u) {
-                    if constexpr (GATED) {
+                    if constexpr (GB) {
                         if (u >= u0 && u < u1) emit_row(u, b[u]);
                     } else {
                         Row o;
@@ -492,7 +540,7 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                         Row r;
                         r.load(lpx + decltype(u_c)::value * SH::CB_BYTES);
                         add_sq(r);
-                        if constexpr (GATED) {      // h = u * silu(g) is finite when u and g are (up to overflow, see above)
+                        if constexpr (GB) {         // h = u * silu(g) is finite when u and g are (up to overflow, see above)
                             r.load(lpx + SH::X_BYTES + decltype(u_c)::value * SH::CB_BYTES);
                             add_sq(r);
                         }
@@ -614,6 +662,14 @@ dwconv_bwd_split_gated_kernel(const void* __restrict__ z, const void* __restrict
         split_role<BF16, K, VEC, RW, NRG, NCW, false, 0, true>(dy, z, cu, w, nullptr, dz, partial, g);
     else
         split_role<BF16, K, VEC, RW, NRG, NCW, false, 1, true>(dy, z, cu, w, nullptr, dz, partial, g);
+}
+
+// x = z = [u | g] [T, 2C]: y = bias + conv(u * silu(g))
+template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>
+__global__ void __launch_bounds__(NCW * NRG * 64)
+dwconv_fwd_split_gated_kernel(const void* __restrict__ z, const int32_t* __restrict__ cu, const void* __restrict__ w,
+                              const void* __restrict__ bias, void* __restrict__ y, const LdsGeo g) {
+    split_role<BF16, K, VEC, RW, NRG, NCW, true, 0, true>(z, nullptr, cu, w, bias, y, nullptr, g);
 }
 
 template <bool BF16, int K, int VEC, int RW, int NRG, int NCW>

@@ -55,9 +55,10 @@ LENS_LONG = LENS_MIX + [40, 33, 31, 30, 29, 16, 15, 14, 0, 1, 1, 700]
                                        (torch.float32, torch.float32, 776), (torch.bfloat16, torch.bfloat16, 1152)])
 def test_long_gated_kernel_sizes_and_widths(K, dt, wdt, C):
     """K = 15 and 31 (the intermediate-width configuration is C = 2048, K = 31): the forward forms the gate product in
-    LDS once per staged element; the backward is the role-split kernel with the gate in both roles (rows of at least
-    512 bytes) or the sliding-window kernel with the gate on its centre rows (C = 256 in bf16 would be; 520 takes
-    two column blocks, the second nearly empty)."""
+    LDS once per staged element (rows of at least 512 bytes: every wave gates its share of a 128-row tile and then runs
+    the taps; narrower rows: loader waves gate 32-row tiles); the backward is the role-split kernel with the gate in
+    both roles (rows of at least 512 bytes) or the sliding-window kernel with the gate on its centre rows (C = 256 in
+    bf16 would be; 520 takes column blocks of which the last is nearly empty)."""
     print(f"[case] long gated K={K} C={C} {dt} w {wdt}", flush=True)
     _check(*_case(LENS_LONG, C, K, dt, wdt, seed=K + C), f"gated K={K} C={C} {dt}")
     _check(*_case(LENS_LONG[::-1], C, K, dt, wdt, seed=K + C + 1), f"gated residual K={K} C={C} {dt}", residual=True)
@@ -99,6 +100,30 @@ def test_nonfinite_gate_inputs_reach_only_the_taps_their_products_belong_to(C, K
         assert bool((~torch.isfinite(dw[:, touched])).all()), f"{what}: a tap the rows feed stayed finite"
         assert torch.equal(dw[:, ~touched], dw0[:, ~touched]), f"{what}: a tap the rows do not feed changed"
         assert torch.equal(db, db0), f"{what}: db changed"
+
+
+@pytest.mark.parametrize("C,K,dt", [(2048, 31, torch.bfloat16), (1024, 15, torch.bfloat16), (512, 31, torch.float32),
+                                     (1024, 7, torch.bfloat16)])
+def test_gated_forward_keeps_nonfinite_rows_inside_their_sequence(C, K, dt):
+    """The forward at K = 15 and 31 turns whole staged tiles, halo rows of neighbouring sequences included, into
+    h = x_proj * silu(gate) in LDS before any tap is taken: an Inf or NaN there must stay out of every other sequence's
+    rows (taps across a boundary are skipped, never multiplied by zero), which must come out bit for bit as without it."""
+    lens = [40, 1, 2, 50, 1, 300, 2, 30, 7, 1, 213, 2, 64, 1, 33, 700, 2, 1, 129, 127]
+    z, cu, w, b, dy = _case(lens, C, K, dt, dt, seed=C + K + 3)
+    cul = cu.tolist()
+    zd, cud, wd, bd = (t.to(DEV) for t in (z, cu, w, b))
+    y0 = npa.gated_dwconv_fwd(zd, cud, wd, bd)
+    for what, pick, col0, val in (("Inf in x_proj", lambda i, n: n <= 2, 0, float("inf")),
+                                  ("NaN in gate", lambda i, n: i % 3 == 0, C, float("nan"))):
+        z2 = z.clone()
+        poisoned = torch.zeros(z.shape[0], dtype=torch.bool)
+        for i, n in enumerate(lens):
+            if pick(i, n):
+                z2[cul[i]:cul[i + 1], col0:col0 + C] = val
+                poisoned[cul[i]:cul[i + 1]] = True
+        y = npa.gated_dwconv_fwd(z2.to(DEV), cud, wd, bd).cpu()
+        assert torch.equal(y[~poisoned], y0.cpu()[~poisoned]), f"{what}: a row of another sequence changed"
+        assert bool((~torch.isfinite(y[poisoned].float())).all()), f"{what}: a row of a poisoned sequence stayed finite"
 
 
 @pytest.mark.parametrize("C,K", [(1024, 7), (2048, 31), (100, 7)])
