@@ -1286,25 +1286,33 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
         return;
     }
     // ---- block-level pass: sum the NRG row groups of each wave-column, group order 0,1,2,... ----
-    // (the tiles are dead after the last barrier above; loader waves only keep the barriers company)
-    float* red = reinterpret_cast<float*>(lds_raw);   // [NWC][VEC][64]
+    // The tiles are dead after the last barrier above. Every wave of row groups 1.. leaves all its sums in LDS, one
+    // barrier, and the waves of row group 0 add them up and write the slab (one barrier for the whole pass: a barrier
+    // per tap would also wait for the slab stores of the tap before, which end the kernel of every block at once).
+    constexpr int NV = K + 1 + (NORM ? 2 : 0);
+    static_assert((long long)NV * SH::NWC * VEC * 256 <= 2LL * BUF_BYTES, "the sums of all compute waves fit the dead tiles");
+    float* red = reinterpret_cast<float*>(lds_raw);   // [NV][NWC][VEC][64]
+    auto sum_of = [&](int kk, int v) __attribute__((always_inline)) {
+        return (kk < K) ? dwa[v][kk < K ? kk : 0] : (kk == K) ? dba[v] : (kk == K + 1) ? dga[NORM ? v : 0] : dbb[NORM ? v : 0];
+    };
+    if (!is_loader && rg > 0) {
 #pragma unroll
-    for (int kk = 0; kk <= K + (NORM ? 2 : 0); ++kk) {
-        float val[VEC];
+        for (int kk = 0; kk < NV; ++kk)
 #pragma unroll
-        for (int v = 0; v < VEC; ++v)
-            val[v] = (kk < K) ? dwa[v][kk < K ? kk : 0] : (kk == K) ? dba[v] : (kk == K + 1) ? dga[NORM ? v : 0] : dbb[NORM ? v : 0];
-        if (!is_loader && rg > 0) {
+            for (int v = 0; v < VEC; ++v) red[((kk * SH::NWC + wv) * VEC + v) * 64 + lane] = sum_of(kk, v);
+    }
+    __syncthreads();
+    if (!is_loader && rg == 0) {
 #pragma unroll
-            for (int v = 0; v < VEC; ++v) red[(wv * VEC + v) * 64 + lane] = val[v];
-        }
-        __syncthreads();
-        if (!is_loader && rg == 0) {
+        for (int kk = 0; kk < NV; ++kk) {
+            float val[VEC];
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) val[v] = sum_of(kk, v);
 #pragma unroll
             for (int j = 1; j < NRG; ++j) {
                 const int ow = j * NCW + wc;
 #pragma unroll
-                for (int v = 0; v < VEC; ++v) val[v] += red[(ow * VEC + v) * 64 + lane];
+                for (int v = 0; v < VEC; ++v) val[v] += red[((kk * SH::NWC + ow) * VEC + v) * 64 + lane];
             }
             if (active) {
                 float* dst = kk <= K ? slab + (size_t)kk * C + c0 : ln.partial2 + ((size_t)tb * 2 + (kk - K - 1)) * C + c0;
@@ -1312,7 +1320,6 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                 for (int v = 0; v < VEC; ++v) dst[v] = val[v];
             }
         }
-        __syncthreads();
     }
 }
 
