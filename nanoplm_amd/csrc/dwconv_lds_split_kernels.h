@@ -30,8 +30,12 @@
 // of the sequence (zero for the others), skips chunks of staged rows that hold none of the sequence's and masks
 // single rows of another sequence inside a chunk (the mask rides on the bf16 -> fp32 conversion).
 //
+// The forward at these kernel sizes is the dx role alone on all 16 waves (taps in forward order, the bias as the row
+// sums' start). Its gated form (input z = [u | g], conv over h = u * silu(g)) stages a u tile and a g tile, has the 16
+// waves turn them into one fp32 h tile in place once per staged element, and runs the same schedules over that.
+//
 // No counterpart in the reference (peymanvahidi/nanoplm 0.1.6 has no convolution); tensor contract:
-// modeling.py:339,421-439 and collator.py:322-325,405-458.
+// modeling.py:339,421-439 and collator.py:322-325,405-458 (the gate product: modeling.py:300-302).
 #pragma once
 #include "dwconv_lds_kernels.h"
 
