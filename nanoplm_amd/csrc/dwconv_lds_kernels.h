@@ -258,6 +258,31 @@ __device__ __forceinline__ bool wave_locate(SeqCursor& sc, int& nce, CU cu, int 
     if (!in) nce = (sc.seq + 1 < S) ? cu_at(cu, sc.seq + 2) : T;
     return in;
 }
+// wave_locate through a row whose sequence index is already known: `lo` is what SeqCursor::locate finds for row
+// `anchor` <= tf (the first i in [0, S) with cu[i+1] > anchor, else S). cu[lo], cu[lo+1] and cu[lo+2] (indices clamped
+// to S) are three independent scalar loads behind one wait, where the binary search is a chain of log2(S) dependent
+// ones; the cursor then steps from the anchor's sequence to that of row tf (no step when both lie in one sequence).
+template <int RW, int P>
+__device__ __forceinline__ bool wave_locate_from(SeqCursor& sc, int& nce, const int32_t* __restrict__ cu, int S, int T, int anchor,
+                                                 int tf, int lo) {
+    if (tf >= T) return true;
+    const int32_t* p0 = cu + (lo < S ? lo : S);
+    const int32_t* p1 = cu + (lo + 1 < S ? lo + 1 : S);
+    const int32_t* p2 = cu + (lo + 2 < S ? lo + 2 : S);
+    int c0, c1, c2;
+    asm volatile("s_load_dword %0, %3, 0x0\n\ts_load_dword %1, %4, 0x0\n\ts_load_dword %2, %5, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(c0), "=&s"(c1), "=&s"(c2) : "s"(p0), "s"(p1), "s"(p2) : "memory");
+    sc.seq = lo;
+    sc.cs = c0;                                  // cu[lo], or cu[S] for rows at or after the last sequence's end
+    sc.ce = lo < S ? c1 : T;
+    if (sc.cs > anchor) { sc.ce = sc.cs; sc.cs = 0; sc.seq = -1; }   // the anchor lies before cu[0]
+    const bool stepped = tf >= sc.ce && sc.seq < S;
+    sc.advance(ScalarCu{cu}, S, T, tf);
+    const int tl = (tf + RW - 1 < T) ? tf + RW - 1 : T - 1;
+    const bool in = (tf - P >= sc.cs) && (tl + P < sc.ce);
+    if (!in) nce = (sc.seq + 1 >= S) ? T : (!stepped && sc.seq == lo) ? c2 : cu_at(ScalarCu{cu}, sc.seq + 2);
+    return in;
+}
 // SeqCursor::advance that takes its first step from the prefetched `nce` (valid while `fresh`).
 template <typename CU>
 __device__ __forceinline__ void advance_prefetched(SeqCursor& sq, int nce, bool& fresh, CU cu, int S, int T, int t) {

@@ -70,7 +70,8 @@ struct SplitShape {
     static constexpr int IN_BYTES = NROWS * CB_BYTES;      // dy tile
     static constexpr int X_BYTES = FWD ? 0 : R * CB_BYTES; // backward: x tile, no halo (gated: the u tile, and as much again for g)
     static constexpr int BUF_BYTES = GF ? 2 * IN_BYTES : IN_BYTES + X_BYTES * (GATED ? 2 : 1);
-    static constexpr int LDS_BYTES = 2 * BUF_BYTES;
+    static constexpr int TAB_TILES = 64;                   // tiles of a block whose sequence index is looked up ahead
+    static constexpr int LDS_BYTES = 2 * BUF_BYTES + TAB_TILES * 4;   // two tile buffers and that table
     static constexpr int RPL = 64 / CPR;                   // staged rows per 1 KiB load (64 lanes x 16 bytes)
     static constexpr int NLD_IN = (NROWS + RPL - 1) / RPL; // loads of a dy tile
     static constexpr int NLD_X1 = FWD ? 0 : (R + RPL - 1) / RPL;  // loads of an x tile (gated: of the u tile, of the g tile)
@@ -78,7 +79,7 @@ struct SplitShape {
     static constexpr int ROW_UNITS = NROWS * NCW;          // gated forward: (staged row, wave-column) pairs to gate
     static_assert(CB_BYTES == 256 || CB_BYTES == 512 || CB_BYTES == 1024, "a staged row is 16, 32 or 64 chunks");
     static_assert(NW <= 16, "at most 1024 threads per block");
-    static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers must fit in LDS");
+    static_assert(LDS_BYTES <= kLdsBytes, "two tile buffers and the table must fit in LDS");
     static_assert(NJ * CB_BYTES <= 65536, "ds_read immediate offsets (a wave reads NJ rows from one base) are 16 bit");
     static_assert(NW * VEC * 64 * 4 <= LDS_BYTES, "the final reduction reuses the tile buffers");
     static_assert(NW == 16, "4 waves per SIMD and one block per CU");
@@ -262,6 +263,33 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
     if constexpr (LOADS) {
         stage_begin(lds_raw, tb * R);
         for (int n = 0; n < NPW; ++n) stage_one(n);
+    }
+    // Entry l of seq_tab: the sequence index (what the binary search of SeqCursor::locate returns) of the first row of
+    // the block's tile in round l, for the first TAB_TILES rounds: 64 searches side by side on the lanes of wave 0, once.
+    // The lookup of the next tile at the end of every tile is then three independent scalar loads (wave_locate_from) and
+    // not a chain of log2(S) dependent ones on which all 16 waves of the block wait at the same time, with nothing else
+    // to issue (measured per wave and 64-row tile of the backward at T=131072, C=2048, 418 sequences: 1100-1400 of 13900
+    // cycles). The table lives in LDS behind the tile buffers: as a register it would be live across the row schedules.
+    // With a handful of sequences the binary search is two or three steps and stays (one long sequence, backward at
+    // T=131072, C=2048: 457 us with it, 465 us through the table; 418 sequences: 498-518 against 489-497 us).
+    typedef volatile __attribute__((address_space(3))) int32_t lds_i32;
+    lds_i32* seq_tab = (lds_i32*)(lds_raw + 2 * SH::BUF_BYTES);
+    const bool use_tab = S >= 16;
+    if (use_tab && wv == 0) {
+        int t = T;
+        if (lane < ntl) {
+            const int q_ = (int)(((long long)tb + (long long)lane * g.rot_step) % g.nbt);     // lds_next_slot, lane times
+            const int tile = lane * g.nbt + q_;
+            if (tile < g.ntiles) t = tile * R;
+        }
+        int lo = 0, hi = S;     // first i in [0, S) with cu[i + 1] > t, else S
+        while (__builtin_amdgcn_ballot_w64(lo < hi) != 0) {
+            if (lo < hi) {
+                const int mid = (lo + hi) >> 1;
+                if (cu[mid + 1] > t) hi = mid; else lo = mid + 1;
+            }
+        }
+        seq_tab[lane] = lo;     // visible to the block after the barrier below
     }
     SeqCursor sc;
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
@@ -609,7 +637,12 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
                 }
             }
         }
-        if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cu, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+        if (it + 1 < ntl) {
+            if (use_tab && it + 1 < SH::TAB_TILES)
+                interior = wave_locate_from<RW, P>(sc, nce, cu, S, T, rn, rn + rg * RW, __builtin_amdgcn_readfirstlane(seq_tab[it + 1]));
+            else
+                interior = wave_locate<RW, P>(sc, nce, cu, S, T, rn + rg * RW);
+        }
         if constexpr (LOADS) wait_vmem_all();   // this wave's share of the next tile has landed
         __syncthreads();   // so has everybody else's; this tile's buffer may be overwritten
         q = qn;
