@@ -55,13 +55,13 @@ MEASURED_TRAFFIC = {
     ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136263218,                       # 1.015 x algorithmic
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544056884,                   # 1.013 x
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816854701,                  # 1.014 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1075067450,       # 1.001 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619771871,      # 1.005 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1076345885,       # 1.002 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619855210,      # 1.005 x
     ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272190087,    # 1.014 x
     ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410652860,   # 1.020 x
     # --gated --config 4 (profiles/bench_cfg4_gated_hbm_traffic.md)
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1618986278,    # 1.006 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693480516,   # 1.003 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1635827018,    # 1.016 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693555429,   # 1.003 x
     # --ln and --fp32 --ln (profiles/bench_cfg3_layernorm_fused_hbm_traffic.md); the backward figure is the fused kernel's alone
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551574918,             # 1.027 x
     ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830259811,            # 1.031 x
