@@ -868,6 +868,41 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
     sc.seq = 0; sc.cs = 0; sc.ce = 0;
     bool interior = true;
     int nce = 0;
+    // WHOLE: the sequence index of the first row of the block's tile in each of its first 64 rounds, found by 64 binary
+    // searches side by side on the lanes of wave 0 and left in LDS behind the row statistics: the lookup of a wave's next
+    // tile, which sits in every wave's chain from the taps to the row sums, is then one LDS read and three independent
+    // scalar loads (wave_locate_from) instead of log2(S) dependent ones. With a handful of sequences the search stays.
+    constexpr int TAB_TILES = 64;
+    typedef volatile __attribute__((address_space(3))) int32_t lds_i32;
+    lds_i32* seq_tab = (lds_i32*)(lds_raw + 2 * BUF_BYTES + RED_BYTES + 2 * R * 8);
+    const bool use_tab = WHOLE && S >= 16;
+    if constexpr (WHOLE) {
+        if (use_tab && wv == 0) {
+            int t = T;
+            if (lane < ntl) {
+                const int q_ = (int)(((long long)tb + (long long)lane * g.rot_step) % g.nbt);     // lds_next_slot, lane times
+                const int tile = lane * g.nbt + q_;
+                if (tile < g.ntiles) t = tile * R;
+            }
+            int lo = 0, hi = S;     // first i in [0, S) with cu[i + 1] > t, else S
+            while (__builtin_amdgcn_ballot_w64(lo < hi) != 0) {
+                if (lo < hi) {
+                    const int mid = (lo + hi) >> 1;
+                    if (cu[mid + 1] > t) hi = mid; else lo = mid + 1;
+                }
+            }
+            seq_tab[lane] = lo;     // visible to the block after the barrier below
+        }
+    }
+    // the boundary lookup of the wave's tile in round it + 1
+    auto locate_next = [&](int it, int qn) __attribute__((always_inline)) {
+        const int rn = lds_tile_row0(g, it + 1, qn, R);
+        if constexpr (WHOLE) {
+            if (use_tab && it + 1 < TAB_TILES)
+                return wave_locate_from<RW, P>(sc, nce, cu, S, T, rn, rn + rg * RW, __builtin_amdgcn_readfirstlane(seq_tab[it + 1]));
+        }
+        return wave_locate<RW, P>(sc, nce, cuq, S, T, rn + rg * RW);
+    };
     if (!is_loader) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, tb * R + rg * RW);
     __syncthreads();
 
@@ -951,7 +986,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                         // The boundary lookup for the next tile (a chain of dependent scalar loads) goes here, between the
                         // taps and the row sums, where the other waves of the SIMD are at their arithmetic and not, as at
                         // the end of the tile, all at the same chain.
-                        if (it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+                        if (it + 1 < ntl) interior = locate_next(it, qn);
                         located = true;
                     }
                     if constexpr (WDX) {
@@ -1282,7 +1317,7 @@ dwconv_bwd_lds_kernel(const void* __restrict__ x, const void* __restrict__ dy, c
                     }
                 }
             }
-            if (!located && it + 1 < ntl) interior = wave_locate<RW, P>(sc, nce, cuq, S, T, lds_tile_row0(g, it + 1, qn, R) + rg * RW);
+            if (!located && it + 1 < ntl) interior = locate_next(it, qn);
         }
         // SELF: every wave has waited for its share of the next tile before it stored dx, so the stores need not be
         // acknowledged before the tile changes hands (__syncthreads() would wait for them)
