@@ -63,10 +63,10 @@ MEASURED_TRAFFIC = {
     ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1635827018,    # 1.016 x
     ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693555429,   # 1.003 x
     # --ln and --fp32 --ln (profiles/bench_cfg3_layernorm_fused_hbm_traffic.md); the backward figure is the fused kernel's alone
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551574918,             # 1.027 x
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830259811,            # 1.031 x
-    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "forward", "ln"): 1092335114,            # 1.017 x
-    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "backward", "ln"): 1641586548,           # 1.019 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551581056,             # 1.027 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830319410,            # 1.031 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "forward", "ln"): 1092089122,            # 1.017 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "backward", "ln"): 1641722624,           # 1.019 x
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
