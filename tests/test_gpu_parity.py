@@ -493,6 +493,40 @@ LENS_SPLIT = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4, 15, 1
               29, 0, 0, 45, 1200, 14]
 
 
+@pytest.mark.parametrize("K,C,dt,nbt", [(31, 256, torch.bfloat16, 1), (31, 256, torch.bfloat16, 2), (15, 512, torch.bfloat16, 1),
+                                        (31, 128, torch.float32, 1), (15, 128, torch.float32, 3)])
+def test_role_split_blocks_that_walk_more_than_64_tiles(K, C, dt, nbt):
+    """A block looks up the sequence of its next tile in a table it fills for its first 64 rounds and by a binary search
+    after that; with at least 16 sequences (fewer: always the search). One to three blocks over 11388 rows walk 178, 89
+    and 60 backward tiles of 64 rows and 89, 45 and 30 forward tiles of 128 rows each: both sides of that switch, in both
+    passes. y and dx equal the sliding-window kernels' bit for bit, everything the oracle's."""
+    print(f"[case] K={K} C={C} {dt} nbt={nbt}", flush=True)
+    x, cu, w, b, dy = _random_case(LENS_SPLIT * 4, C, K, dt, dt, seed=C + nbt + K)
+    assert x.shape[0] == 11388 and cu.numel() - 1 >= 16
+    xd, cud, wd, dyd, bd = x.to(DEV), cu.to(DEV), w.to(DEV), dy.to(DEV), b.to(DEV)
+    y1 = npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=_lib.Tuning(algo=1))
+    y3 = npa.varlen_dwconv_fwd(xd, cud, wd, bd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    assert torch.equal(y3, y1)
+    assert_act_close(y3, O.c_oracle_fwd(x, cu, w, b), dt, "y")
+    dx64, dw64, db64 = O.c_oracle_bwd(x, dy, cu, w)
+    dx1, dw1, db1 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=1))
+    dx3, dw3, db3 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    assert torch.equal(dx3, dx1)
+    assert_act_close(dx3, dx64, dt, "dx")
+    assert_red_close(dw3, dw64, "dw")
+    assert_red_close(db3, db64, "db")
+    # the same rows as fewer than 16 sequences (the search in every round): neighbours merged, same total
+    lens = torch.tensor(LENS_SPLIT * 4).view(-1, 14).sum(1).tolist()
+    cu2 = cu_from_lengths(torch.tensor(lens))
+    assert cu2.numel() - 1 == 10 and int(cu2[-1]) == x.shape[0]
+    dx64b, dw64b, db64b = O.c_oracle_bwd(x, dy, cu2, w)
+    dxb, dwb, dbb = npa.varlen_dwconv_bwd(xd, dyd, cu2.to(DEV), wd, tuning=_lib.Tuning(algo=3, nbt=nbt))
+    assert torch.equal(dxb, npa.varlen_dwconv_bwd(xd, dyd, cu2.to(DEV), wd, tuning=_lib.Tuning(algo=1))[0])
+    assert_act_close(dxb, dx64b, dt, "dx, 10 sequences")
+    assert_red_close(dwb, dw64b, "dw, 10 sequences")
+    assert_red_close(dbb, db64b, "db, 10 sequences")
+
+
 @pytest.mark.parametrize("C,dt", [(256, torch.bfloat16), (264, torch.bfloat16), (1024, torch.bfloat16),
                                   (1152, torch.bfloat16), (2048, torch.bfloat16), (2056, torch.bfloat16),
                                   (128, torch.float32), (388, torch.float32), (1024, torch.float32)])
