@@ -17,6 +17,13 @@
  *   with [s(t), e(t)) the cu interval that contains row t. Taps never cross a sequence boundary
  *   (masked by selection, so a NaN/Inf in one sequence cannot reach another).
  *
+ *   Kernel sizes: K = 3, 5, 7, 9, 15 and 31 have kernels of their own. Any other odd K <= 31 runs on the
+ *   kernels of the next of 3, 15, 31 with zero taps on either side (w and dw keep rows of K taps; the
+ *   workspace holds slabs of that size): for finite inputs the same sums with exact zeros added, so the
+ *   same results; a NaN/Inf in x or dy then reaches the rows within that larger half-width of its own
+ *   sequence (0 * Inf), never another sequence, and never a tap of dw that its products do not belong
+ *   to. Odd K from 33 to NPLM_DWCONV_MAX_K run untuned kernels (one wave per row).
+ *
  * Where this sits in the reference (peymanvahidi/nanoplm 0.1.6): the reference snapshot holds no
  * convolution; the ABI binds at the call site a conv module would occupy on the packed path,
  * src/nanoplm/pretraining/models/modern_bert/modeling.py:421-439 (encoder layer over x:[T,hidden]

@@ -36,6 +36,10 @@ constexpr int kMaxTileRows = 1 << 16;
 constexpr size_t kSlabBudgetBytes = 16u << 20;   // cap on dw/db partials (written once, read once)
 
 bool specialised_k(int K) { return K == 3 || K == 5 || K == 7 || K == 9 || K == 15 || K == 31; }
+// The kernel size a plain conv of K taps runs as: an odd K below 31 without kernels of its own takes the next size that
+// has them, with (exec - K) / 2 zero taps on either side (W_TAP_OFF_SHIFT); the caller's weight and dw rows stay K long.
+// Runtime-K kernels (one wave per row) remain for K > 31.
+int exec_kernel_size(int K) { return K > 31 || specialised_k(K) ? K : K < 3 ? 3 : K < 15 ? 15 : 31; }
 
 int pow2_floor(int v) { int p = 1; while (p * 2 <= v) p *= 2; return p; }
 int ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
@@ -397,7 +401,9 @@ int fwd_impl(const void* x, const int32_t* cu, const void* w, const void* b, voi
     if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
     if (T == 0) return 0;
     if (!x || !cu || !w || !y) return -NPLM_DWCONV_ENULL;
-    const int w_flags = kernel_w_flags(w_dtype, flags);
+    const int tap_off = (exec_kernel_size(K) - K) / 2;
+    K = exec_kernel_size(K);        // from here on the kernel size that runs
+    const int w_flags = kernel_w_flags(w_dtype, flags) | (tap_off << W_TAP_OFF_SHIFT);
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t E = bf16 ? 2 : 4;
     const uintptr_t bits = (uintptr_t)x | (uintptr_t)y;
@@ -452,7 +458,6 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     int rc = check_common(T, C, K, S, act_dtype, w_dtype);
     if (rc) return rc;
     if (flags & ~(uint32_t)(NPLM_DWCONV_RESIDUAL | NPLM_DWCONV_GRADS_BF16)) return -NPLM_DWCONV_EFLAGS;
-    const int w_flags = kernel_w_flags(w_dtype, flags);
     const int out_bf16 = (flags & NPLM_DWCONV_GRADS_BF16) ? 1 : 0;      // dw, db are bf16 buffers
     hipStream_t s = (hipStream_t)stream;
     const bool want_red = dw || db;
@@ -461,6 +466,9 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         if (e == hipSuccess) e = out_bf16 ? fill_zero16(db, C, s) : fill_zero(db, C, s);
         return (int)e;
     }
+    const int tap_off = (exec_kernel_size(K) - K) / 2;
+    K = exec_kernel_size(K);        // from here on the kernel size that runs (slabs of K + 1 rows; dw rows stay the caller's)
+    const int w_flags = kernel_w_flags(w_dtype, flags) | (tap_off << W_TAP_OFF_SHIFT);
     if (!dx && !want_red) return 0;
     if (!dy || !cu || !w || (want_red && !x)) return -NPLM_DWCONV_ENULL;
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
@@ -495,7 +503,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         }
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0,
-                           s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
+                           s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16, tap_off);
         return (int)hipGetLastError();
     }
     if (algo == 2) {
@@ -521,7 +529,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
         if (want_red) {
             const long long n_out = (long long)(K + 1) * C;
             hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)),
-                               dim3(64 * FIN_SPLIT), 0, s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
+                               dim3(64 * FIN_SPLIT), 0, s, (const float*)part, lp.nbt, C, K, dw, db, out_bf16, tap_off);
             e = hipGetLastError();
         }
         return (int)e;
@@ -586,7 +594,7 @@ int bwd_impl(const void* x, const void* dy, const int32_t* cu, const void* w, vo
     if (want_red) {
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)partial, p.nbt, C, K, dw, db, out_bf16);
+                           (const float*)partial, p.nbt, C, K, dw, db, out_bf16, tap_off);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
@@ -979,7 +987,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
+                           (const float*)part, lp.nbt, C, K, dw, db, out_bf16, 0);
         return (int)hipGetLastError();
     }
     if (long_gated_bwd_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
@@ -998,7 +1006,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, p.nbt, C, K, dw, db, out_bf16);
+                           (const float*)part, p.nbt, C, K, dw, db, out_bf16, 0);
         return (int)hipGetLastError();
     }
     if (!gated_supported(true, bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
@@ -1023,7 +1031,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     if (e != hipSuccess) return (int)e;
     const long long n_out = (long long)(K + 1) * C;
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, lp.nbt, C, K, dw, db, out_bf16);
+                       (const float*)part, lp.nbt, C, K, dw, db, out_bf16, 0);
     return (int)hipGetLastError();
 }
 
@@ -1064,6 +1072,7 @@ int nplm_dwconv_fwd_tuned(const void* x, const int32_t* cu, const void* w, const
 
 size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    K = exec_kernel_size(K);        // the slabs have the rows of the kernel size that runs
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     // enough for whichever kernel family the library picks for these sizes (the choice also depends
     // on pointer alignment, which is not known here)
@@ -1084,6 +1093,7 @@ size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t 
 
 int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    K = exec_kernel_size(K);
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const int algo = choose_algo(true, tune, bf16, T, C, K, 0);
     if (algo < 0) return 0;

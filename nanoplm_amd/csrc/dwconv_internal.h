@@ -46,7 +46,8 @@ int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, cons
                           float* dw, float* db, void* workspace, size_t workspace_bytes, int64_t T,
                           int32_t C, int32_t K, int32_t S, int32_t act_dtype, int32_t w_dtype,
                           void* stream, const nplm_dwconv_tuning* tune);
-// Token-blocks (= workspace slabs of (K+1)*C floats) a backward launch with these overrides uses.
+// Token-blocks (= workspace slabs of (K'+1)*C floats, K' the kernel size that runs: K, or for an odd K <= 31 without
+// kernels of its own the next of 3, 15, 31) a backward launch with these overrides uses.
 int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune);
 
 // Host-side run of the kernels' boundary cursor (SeqCursor) over a HOST copy of cu: for rows

@@ -61,13 +61,28 @@ __device__ __forceinline__ void block_coords(const Geo& g, int& cb, int& tb) {
 // Bits of the w_flags launch parameter.
 constexpr int W_BF16 = 1;      // weights and bias are bf16 (otherwise fp32)
 constexpr int W_RESIDUAL = 2;  // compute x + conv(x) (forward) / dy + conv^T(dy) (dx)
+// A kernel built for K taps also runs a conv of K - 2 * off taps (the caller's weight rows are that long): taps
+// off .. K-1-off carry the caller's weights, the outer ones are zero, and the reduction writes the inner rows of dw only.
+constexpr int W_TAP_OFF_SHIFT = 8;
+__host__ __device__ constexpr int w_tap_off(int w_flags) { return (w_flags >> W_TAP_OFF_SHIFT) & 0xff; }
 
 // Weights of channels c0 .. c0+VEC-1 as fp32 registers. The fused residual costs nothing: the centre
 // tap is valid for every row, so x + conv(x; w) = conv(x; w + delta_centre); one is added to the
 // centre weight here (exact for bf16 weights, one fp32 rounding otherwise). dw does not read wr.
 template <int VEC, int K>
 __device__ __forceinline__ void load_weights(const void* __restrict__ w, int w_flags, int c0, float (&wr)[VEC][K]) {
-    if (w_flags & W_BF16) {
+    if (const int off = w_tap_off(w_flags); off != 0) {      // weight rows of K - 2 * off taps
+        const int kw = K - 2 * off;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const int r = k - off;
+                const size_t i = (size_t)(c0 + v) * kw + (r >= 0 && r < kw ? r : 0);
+                const float t = (w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[i]) : reinterpret_cast<const float*>(w)[i];
+                wr[v][k] = (r >= 0 && r < kw) ? t : 0.f;
+            }
+    } else if (w_flags & W_BF16) {
         const uint16_t* wp = reinterpret_cast<const uint16_t*>(w) + (size_t)c0 * K;
 #pragma unroll
         for (int v = 0; v < VEC; ++v)
@@ -497,9 +512,11 @@ constexpr int FIN_SPLIT = 16;
 
 // One block of the reduction: 64 consecutive (tap, channel) outputs, SPLIT groups of slabs summed in LDS.
 // out_bf16: dw and db are bf16 buffers (the fp32 totals are rounded once, nearest-even, on store).
+// tap_off: dw has rows of K - 2 * tap_off taps, slab rows tap_off .. K-1-tap_off (see W_TAP_OFF_SHIFT).
 template <int SPLIT>
 __device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int block, const float* __restrict__ partial, int nbt, int C,
-                                               int K, float* __restrict__ dw, float* __restrict__ db, int out_bf16 = 0) {
+                                               int K, float* __restrict__ dw, float* __restrict__ db, int out_bf16 = 0,
+                                               int tap_off = 0) {
     const int lane = (int)(threadIdx.x & 63);
     const int grp = (int)(threadIdx.x >> 6);
     const long long n_out = (long long)(K + 1) * C;
@@ -530,11 +547,13 @@ __device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int bloc
         for (int g = 1; g < SPLIT; ++g) tot += red[g][lane];
         const int kk = (int)(o / C);
         const int c = (int)(o - (long long)kk * C);
+        const int kw = K - 2 * tap_off, r = kk - tap_off;
+        const bool tap = dw && r >= 0 && r < kw;
         if (out_bf16) {
-            if (kk < K) { if (dw) reinterpret_cast<uint16_t*>(dw)[(size_t)c * K + kk] = f32_to_bf16(tot); }
+            if (kk < K) { if (tap) reinterpret_cast<uint16_t*>(dw)[(size_t)c * kw + r] = f32_to_bf16(tot); }
             else        { if (db) reinterpret_cast<uint16_t*>(db)[c] = f32_to_bf16(tot); }
         } else {
-            if (kk < K) { if (dw) dw[(size_t)c * K + kk] = tot; }
+            if (kk < K) { if (tap) dw[(size_t)c * kw + r] = tot; }
             else        { if (db) db[c] = tot; }
         }
     }
@@ -542,9 +561,10 @@ __device__ __forceinline__ void finalize_block(float (&red)[SPLIT][64], int bloc
 
 template <int SPLIT>
 __global__ void __launch_bounds__(64 * SPLIT) dwconv_finalize_kernel(const float* __restrict__ partial, int nbt, int C, int K,
-                                                                     float* __restrict__ dw, float* __restrict__ db, int out_bf16) {
+                                                                     float* __restrict__ dw, float* __restrict__ db, int out_bf16,
+                                                                     int tap_off) {
     __shared__ float red[SPLIT][64];
-    finalize_block<SPLIT>(red, (int)blockIdx.x, partial, nbt, C, K, dw, db, out_bf16);
+    finalize_block<SPLIT>(red, (int)blockIdx.x, partial, nbt, C, K, dw, db, out_bf16, tap_off);
 }
 
 // Two slab sets of the same launch in one reduction launch (the conv's dw/db and, as a conv of K2 = 1 tap, the

@@ -248,15 +248,32 @@ __device__ __forceinline__ void split_role(const void* __restrict__ in, const vo
         });
     };
     if constexpr (ROLE == 0) {
+        if (const int off = w_tap_off(g.w_flags); off == 0) {
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+#pragma unroll
+                for (int m = 0; m < K; ++m) {
+                    const size_t wi = (size_t)(c0 + v) * K + (FWD ? m : K - 1 - m);
+                    a[v][m] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[wi]) : reinterpret_cast<const float*>(w)[wi];
+                }
+            }
+        } else {        // weight rows of K - 2 * off taps: the outer taps are zero, see W_TAP_OFF_SHIFT
+            const int kw = K - 2 * off;
+#pragma unroll
+            for (int v = 0; v < VEC; ++v) {
+#pragma unroll
+                for (int m = 0; m < K; ++m) {
+                    const int r = (FWD ? m : K - 1 - m) - off;
+                    const bool tap = r >= 0 && r < kw;
+                    const size_t wi = (size_t)(c0 + v) * kw + (tap ? r : 0);
+                    const float t = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[wi]) : reinterpret_cast<const float*>(w)[wi];
+                    a[v][m] = tap ? t : 0.f;
+                }
+            }
+        }
 #pragma unroll
         for (int v = 0; v < VEC; ++v) {
-#pragma unroll
-            for (int m = 0; m < K; ++m) {
-                const size_t wi = (size_t)(c0 + v) * K + (FWD ? m : K - 1 - m);
-                float t = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(w)[wi]) : reinterpret_cast<const float*>(w)[wi];
-                if (m == P && (g.w_flags & W_RESIDUAL)) t += 1.f;
-                a[v][m] = t;
-            }
+            if (g.w_flags & W_RESIDUAL) a[v][P] += 1.f;
             if (FWD && bias) c[v] = (g.w_flags & W_BF16) ? bf16_to_f32(reinterpret_cast<const uint16_t*>(bias)[c0 + v]) : reinterpret_cast<const float*>(bias)[c0 + v];
         }
     }

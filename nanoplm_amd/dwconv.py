@@ -120,6 +120,14 @@ def bwd_workspace_bytes(T: int, C: int, K: int, dtype: torch.dtype) -> int:
     return int(_lib.load().nplm_dwconv_bwd_workspace_bytes(T, C, K, _DTYPES[dtype]))
 
 
+def exec_kernel_size(K: int) -> int:
+    """The kernel size a plain conv of K taps runs as (csrc/dwconv_api.hip::exec_kernel_size): an odd K <= 31 that has no
+    kernels of its own takes the next size that has, with zero taps on either side; its dw/db slabs have that many rows."""
+    if K > 31 or K in (3, 5, 7, 9, 15, 31):
+        return K
+    return 3 if K < 3 else 15 if K < 15 else 31
+
+
 def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, residual: bool = False,
                       tuning: Optional[_lib.Tuning] = None, workspace: Optional[torch.Tensor] = None,
                       grads_bf16: bool = False):
@@ -146,7 +154,7 @@ def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, 
             if tuning is None:
                 nbytes = int(lib.nplm_dwconv_bwd_workspace_bytes(T, C, K, act))
             else:
-                nbytes = int(lib.nplm_dwconv_bwd_slabs(T, C, K, act, tuning)) * (K + 1) * C * 4
+                nbytes = int(lib.nplm_dwconv_bwd_slabs(T, C, K, act, tuning)) * (exec_kernel_size(K) + 1) * C * 4
             workspace = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=x.device)
         stream = dev.stream
         flags = (_lib.RESIDUAL if residual else 0) | (_lib.GRADS_BF16 if grads_bf16 else 0)

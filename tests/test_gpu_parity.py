@@ -163,11 +163,45 @@ def _check_case(x, cu, w, b, dy, what):
 LENS_MIX = [1, 2, 3, 8, 0, 1, 150, 0, 5, 7, 6, 1, 64, 63, 65, 2, 300, 4]
 
 
-@pytest.mark.parametrize("K", [1, 3, 5, 7, 9, 11, 15, 31, 33])
+@pytest.mark.parametrize("K", [1, 3, 5, 7, 9, 11, 13, 15, 17, 21, 29, 31, 33])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float32])
 def test_kernel_sizes(K, dt):
     print(f"[case] K={K} {dt}", flush=True)
     _check_case(*_random_case(LENS_MIX, 256, K, dt, dt, seed=K), f"K={K} {dt}")
+
+
+@pytest.mark.parametrize("K,Kx,C,dt,wdt", [(11, 15, 1024, torch.bfloat16, torch.bfloat16), (13, 15, 264, torch.bfloat16, torch.float32),
+                                           (1, 3, 512, torch.bfloat16, torch.bfloat16), (17, 31, 2048, torch.bfloat16, torch.bfloat16),
+                                           (29, 31, 388, torch.float32, torch.float32), (21, 31, 128, torch.float32, torch.bfloat16)])
+def test_kernel_sizes_without_kernels_of_their_own_run_as_the_next_size_with_zero_taps(K, Kx, C, dt, wdt):
+    """An odd K <= 31 other than 3, 5, 7, 9, 15, 31 is served by the kernels of the next of 3, 15, 31: the caller's [C, K]
+    taps sit in the middle of that kernel's taps and the outer ones are zero. Every output must equal, bit for bit, the
+    call with explicitly zero-padded [C, Kx] taps (dw: its inner K columns), in every kernel family that size has, with
+    and without the fused residual and with gradients stored in bf16; dw / db alone and dx alone take other kernels."""
+    print(f"[case] K={K} as {Kx} C={C} {dt} w {wdt}", flush=True)
+    x, cu, w, b, dy = _random_case(LENS_SPLIT, C, K, dt, wdt, seed=C + K)
+    off = (Kx - K) // 2
+    wx = torch.zeros(C, Kx, dtype=wdt)
+    wx[:, off:off + K] = w
+    xd, cud, wd, wxd, bd, dyd = (t.to(DEV) for t in (x, cu, w, wx, b, dy))
+    _check_case(x, cu, w, b, dy, f"K={K}")
+    algos = [None, 1] + ([2] if Kx == 3 else []) + ([3] if Kx in (15, 31) and (C * (2 if dt == torch.bfloat16 else 4)) % 16 == 0 else [])
+    for algo in algos:
+        tn = None if algo is None else _lib.Tuning(algo=algo)
+        for res in (False, True):
+            assert torch.equal(npa.varlen_dwconv_fwd(xd, cud, wd, bd, residual=res, tuning=tn),
+                               npa.varlen_dwconv_fwd(xd, cud, wxd, bd, residual=res, tuning=tn)), (algo, res)
+            dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, residual=res, tuning=tn)
+            dxx, dwx, dbx = npa.varlen_dwconv_bwd(xd, dyd, cud, wxd, residual=res, tuning=tn)
+            assert dw.shape == (C, K)
+            assert torch.equal(dx, dxx) and torch.equal(dw, dwx[:, off:off + K]) and torch.equal(db, dbx), (algo, res)
+        _, dwb, dbb = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, grads_bf16=True, tuning=tn)
+        assert torch.equal(dwb, dw.bfloat16()) and torch.equal(dbb, db.bfloat16())
+    only_dx = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dw=False)[0]
+    assert torch.equal(only_dx, npa.varlen_dwconv_bwd(xd, dyd, cud, wxd, need_dw=False)[0])
+    _, dw1, db1 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd, need_dx=False)
+    _, dw1x, db1x = npa.varlen_dwconv_bwd(xd, dyd, cud, wxd, need_dx=False)
+    assert torch.equal(dw1, dw1x[:, off:off + K]) and torch.equal(db1, db1x)
 
 
 @pytest.mark.parametrize("C", [1, 7, 8, 24, 64, 72, 100, 128, 130, 384, 520, 576, 640, 768, 1000, 1024, 1152, 1280, 2048,

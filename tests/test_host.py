@@ -12,6 +12,7 @@ import torch
 
 import nanoplm_amd
 from nanoplm_amd import _lib
+from nanoplm_amd.dwconv import exec_kernel_size
 from nanoplm_amd.workloads import cu_from_lengths, make_workload, static_packed_cu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -68,8 +69,10 @@ def test_workspace_bytes_arithmetic():
         # enough for the library's default kernel and for the sliding-window kernel that a request for dx alone or
         # dw/db alone may take instead (K = 31), and no more than the larger of the two
         most = max(slabs, lib.nplm_dwconv_bwd_slabs(T, C, K, act, _lib.Tuning(algo=1)))
-        assert n % 256 == 0 and n >= most * (K + 1) * C * 4 > n - 256
-        assert n <= (16 << 20) + (K + 1) * C * 4       # partials are capped (one slab minimum)
+        Kx = exec_kernel_size(K)        # K = 1 runs as 3 taps and K = 11 as 15, with slabs of that many rows
+        assert Kx == {7: 7, 31: 31, 3: 3, 1: 3, 11: 15}[K]
+        assert n % 256 == 0 and n >= most * (Kx + 1) * C * 4 > n - 256
+        assert n <= (16 << 20) + (Kx + 1) * C * 4       # partials are capped (one slab minimum)
     assert lib.nplm_dwconv_bwd_workspace_bytes(0, 64, 3, 1) == 0
     assert lib.nplm_dwconv_bwd_workspace_bytes(100, 64, 4, 1) == 0
 
