@@ -22,7 +22,8 @@
  *   workspace holds slabs of that size): for finite inputs the same sums with exact zeros added, so the
  *   same results; a NaN/Inf in x or dy then reaches the rows within that larger half-width of its own
  *   sequence (0 * Inf), never another sequence, and never a tap of dw that its products do not belong
- *   to. Odd K from 33 to NPLM_DWCONV_MAX_K run untuned kernels (one wave per row).
+ *   to. Odd K from 33 to NPLM_DWCONV_MAX_K run untuned kernels (one wave per row). The gated entry
+ *   points take the same kernel sizes up to 31 the same way; the LayerNorm-fused ones K = 3, 5, 7, 9 only.
  *
  * Where this sits in the reference (peymanvahidi/nanoplm 0.1.6): the reference snapshot holds no
  * convolution; the ABI binds at the call site a conv module would occupy on the packed path,

@@ -698,6 +698,8 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     if (flags & ~(uint32_t)NPLM_DWCONV_RESIDUAL) return -NPLM_DWCONV_EFLAGS;
     if (T == 0) return 0;
     if (!z || !cu || !w || !y) return -NPLM_DWCONV_ENULL;
+    const int tap_flags = ((exec_kernel_size(K) - K) / 2) << W_TAP_OFF_SHIFT;
+    K = exec_kernel_size(K);        // from here on the kernel size that runs
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if (((uintptr_t)w | (uintptr_t)b) % WE || (uintptr_t)cu % 4) return -NPLM_DWCONV_EALIGN;
@@ -707,7 +709,7 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
         rc = make_split_plan(true, bf16, T, C, K, nullptr, &lp, true);
         if (rc) return rc;
         const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
-        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags) | tap_flags);
         const dim3 grid(lp.ncb * lp.nbt);
         return (int)(K == 31 ? launch_fwd_split_gated_k31(bf16, la, lg, grid, (hipStream_t)stream)
                              : launch_fwd_split_gated_k15(bf16, la, lg, grid, (hipStream_t)stream));
@@ -716,7 +718,7 @@ int nplm_dwconv_gated_fwd(const void* z, const int32_t* cu, const void* w, const
     if (rc) return rc == -NPLM_DWCONV_ETUNING ? -NPLM_DWCONV_EUNSUPPORTED : rc;
     const ConvPtrs la{z, nullptr, cu, w, b, y, nullptr};
     const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4), K);
-    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags) | tap_flags);
     const dim3 grid(lp.ncb * lp.nbt);
     hipStream_t s = (hipStream_t)stream;
     switch (K) {
@@ -936,6 +938,7 @@ int nplm_dwconv_ln_bwd(const void* x, const void* dy, const int32_t* cu, const f
 
 size_t nplm_dwconv_gated_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t act_dtype) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
+    K = exec_kernel_size(K);        // the slabs have the rows of the kernel size that runs
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     if (long_gated_bwd_supported(bf16, T, C, K, 0)) {
         // enough for either kernel: which one runs also depends on pointer alignment, not known here
@@ -970,6 +973,8 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         return (int)e;
     }
     if (!z || !dy || !cu || !w || !dz) return -NPLM_DWCONV_ENULL;
+    const int tap_off = (exec_kernel_size(K) - K) / 2, tap_flags = tap_off << W_TAP_OFF_SHIFT;
+    K = exec_kernel_size(K);        // from here on the kernel size that runs (slabs of K + 1 rows; dw rows stay the caller's)
     const bool bf16 = act_dtype == NPLM_DWCONV_BF16;
     const uintptr_t WE = (w_dtype == NPLM_DWCONV_BF16) ? 2 : 4;
     if ((uintptr_t)w % WE || (uintptr_t)cu % 4 || ((uintptr_t)dw | (uintptr_t)db) % (out_bf16 ? 2 : 4)) return -NPLM_DWCONV_EALIGN;
@@ -981,13 +986,13 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab * (size_t)lp.nbt) return -NPLM_DWCONV_EWORKSPACE;
         float* part = reinterpret_cast<float*>(workspace);
         const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
-        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+        const LdsGeo lg = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags) | tap_flags);
         const dim3 grid(lp.ncb * lp.nbt);
         hipError_t e = K == 31 ? launch_bwd_split_gated_k31(bf16, la, lg, grid, s) : launch_bwd_split_gated_k15(bf16, la, lg, grid, s);
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, lp.nbt, C, K, dw, db, out_bf16, 0);
+                           (const float*)part, lp.nbt, C, K, dw, db, out_bf16, tap_off);
         return (int)hipGetLastError();
     }
     if (long_gated_bwd_supported(bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) {
@@ -998,7 +1003,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (!workspace || (uintptr_t)workspace % 256 || workspace_bytes < slab * (size_t)p.nbt) return -NPLM_DWCONV_EWORKSPACE;
         float* part = reinterpret_cast<float*>(workspace);
         const ConvPtrs a{z, dy, cu, w, nullptr, dz, part};
-        const Geo g = make_geo(p, T, C, S, kernel_w_flags(w_dtype, flags));
+        const Geo g = make_geo(p, T, C, S, kernel_w_flags(w_dtype, flags) | tap_flags);
         const dim3 grid(p.ncb * p.nbt), block(p.bw * p.bt * 64);
         const size_t shmem = (size_t)p.bw * p.bt * p.vec * 64 * sizeof(float);
         hipError_t e = K == 15 ? launch_bwd_gated_k15(bf16, p.unroll, p.maxt, a, g, grid, block, shmem, s)
@@ -1006,7 +1011,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
         if (e != hipSuccess) return (int)e;
         const long long n_out = (long long)(K + 1) * C;
         hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                           (const float*)part, p.nbt, C, K, dw, db, out_bf16, 0);
+                           (const float*)part, p.nbt, C, K, dw, db, out_bf16, tap_off);
         return (int)hipGetLastError();
     }
     if (!gated_supported(true, bf16, T, C, K, (uintptr_t)z | (uintptr_t)dy | (uintptr_t)dz)) return -NPLM_DWCONV_EUNSUPPORTED;
@@ -1019,7 +1024,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     float* part = reinterpret_cast<float*>(workspace);
     const ConvPtrs la{z, dy, cu, w, nullptr, dz, part};
     const bool narrow = lds_gated_narrow((long long)C * (bf16 ? 2 : 4), K);
-    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags));
+    const LdsGeo g = make_lds_geo(lp, T, C, S, kernel_w_flags(w_dtype, flags) | tap_flags);
     const dim3 grid(lp.ncb * lp.nbt);
     hipError_t e = hipErrorInvalidConfiguration;
     switch (K) {
@@ -1031,7 +1036,7 @@ int nplm_dwconv_gated_bwd(const void* z, const void* dy, const int32_t* cu, cons
     if (e != hipSuccess) return (int)e;
     const long long n_out = (long long)(K + 1) * C;
     hipLaunchKernelGGL(dwconv_finalize_kernel<FIN_SPLIT>, dim3((unsigned)((n_out + 63) / 64)), dim3(64 * FIN_SPLIT), 0, s,
-                       (const float*)part, lp.nbt, C, K, dw, db, out_bf16, 0);
+                       (const float*)part, lp.nbt, C, K, dw, db, out_bf16, tap_off);
     return (int)hipGetLastError();
 }
 

@@ -25,7 +25,7 @@ from .dwconv import _DTYPES, _launch_on, _ptr, varlen_dwconv_bwd, varlen_dwconv_
 
 
 def gated_supported(z: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the fused kernels take this call (a kernel size they are built for, rows of C*elemsize >= 1 KiB
+    """Whether the fused kernels take this call (an odd kernel size up to 31, rows of C*elemsize >= 1 KiB
     in multiples of 16 bytes, 16-byte aligned contiguous z on a ROCm device). Informational: the entry
     points below find out from the library's return code."""
     if not (isinstance(z, torch.Tensor) and z.is_cuda and z.dim() == 2 and z.shape[1] % 2 == 0):

@@ -203,10 +203,32 @@ def test_unsupported_shapes_compose_and_the_abi_says_so():
     rc = lib.nplm_dwconv_gated_fwd(zd.data_ptr(), cud.data_ptr(), wd.data_ptr(), None, out.data_ptr(), 48, 100, 7, 3, 1, 1, 0,
                                    torch.cuda.current_stream().cuda_stream)
     assert rc == -_lib.EUNSUPPORTED and "gated" in _lib.strerror(rc)
-    c11 = _case([30, 30], 1024, 11, torch.bfloat16, torch.bfloat16, seed=2)  # K = 11
-    assert not npa.gated_supported(c11[0].to(DEV), c11[2].to(DEV))
-    _composed_case_matches(*c11, "K=11")
-    _composed_case_matches(*_case([30, 7, 30], 512, 13, torch.float32, torch.float32, seed=3), "K=13 fp32")
+    c33 = _case([30, 30], 1024, 33, torch.bfloat16, torch.bfloat16, seed=2)  # K = 33: above the largest built size
+    assert not npa.gated_supported(c33[0].to(DEV), c33[2].to(DEV))
+    _composed_case_matches(*c33, "K=33")
+    _composed_case_matches(*_case([30, 7, 30], 512, 35, torch.float32, torch.float32, seed=3), "K=35 fp32")
+
+
+@pytest.mark.parametrize("K,Kx,C,dt,wdt", [(11, 15, 1024, torch.bfloat16, torch.bfloat16), (13, 15, 256, torch.float32, torch.float32),
+                                           (1, 3, 1152, torch.bfloat16, torch.bfloat16), (21, 31, 2048, torch.bfloat16, torch.float32),
+                                           (29, 31, 520, torch.bfloat16, torch.bfloat16)])
+def test_gated_kernel_sizes_without_kernels_of_their_own_run_as_the_next_size_with_zero_taps(K, Kx, C, dt, wdt):
+    """As for the plain conv: an odd K <= 31 other than 3, 5, 7, 9, 15, 31 runs on the fused gated kernels of the next of
+    3, 15, 31 with zero outer taps; every output equals the call with explicitly padded [C, Kx] taps bit for bit (dw: its
+    inner K columns) and the oracle to the usual tolerances."""
+    print(f"[case] gated K={K} as {Kx} C={C} {dt} w {wdt}", flush=True)
+    z, cu, w, b, dy = _case(LENS_LONG, C, K, dt, wdt, seed=K + C)
+    _check(z, cu, w, b, dy, f"gated K={K} C={C}")
+    off = (Kx - K) // 2
+    wx = torch.zeros(C, Kx, dtype=wdt)
+    wx[:, off:off + K] = w
+    zd, cud, wd, wxd, bd, dyd = (t.to(DEV) for t in (z, cu, w, wx, b, dy))
+    for res in (False, True):
+        assert torch.equal(npa.gated_dwconv_fwd(zd, cud, wd, bd, residual=res), npa.gated_dwconv_fwd(zd, cud, wxd, bd, residual=res))
+        dz, dw, db = npa.gated_dwconv_bwd(zd, dyd, cud, wd, residual=res)
+        dzx, dwx, dbx = npa.gated_dwconv_bwd(zd, dyd, cud, wxd, residual=res)
+        assert dw.shape == (C, K)
+        assert torch.equal(dz, dzx) and torch.equal(dw, dwx[:, off:off + K]) and torch.equal(db, dbx)
 
 
 def test_offset_view_of_z_composes_instead_of_failing():
