@@ -25,7 +25,7 @@ static __device__ __align__(256) unsigned char scratch[NPLM_DWCONV_STATIC_SCRATC
 namespace nplm {
 namespace {
 
-constexpr int kVersion = 101;   // 0.1.1
+constexpr int kVersion = 102;   // 0.1.2: odd kernel sizes up to 31 without kernels of their own run as the next built size
 
 // MI355X: 256 CUs in 8 XCDs. Geometry is a pure function of the problem size so that the
 // reduction order (and with it every output bit) is reproducible.
