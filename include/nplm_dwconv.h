@@ -151,7 +151,8 @@ int nplm_dwconv_bwd_ex(const void* x, const void* dy, const int32_t* cu, const v
  * NPLM_DWCONV_STATIC_SCRATCH_BYTES that lives in the library's own device image, one copy per GPU,
  * held until the process ends. The call allocates and frees nothing. Its first use on a device looks
  * the array's address up (hipGetSymbolAddress) and keeps it, so make one call per device outside any
- * capture. Shapes whose partial sums need more than the array holds (C*(K+1) above 4 Mi elements)
+ * capture. Shapes whose partial sums need more than the array holds (C*(K'+1) above 4 Mi elements,
+ * K' the kernel size that runs, see "Kernel sizes" above)
  * return -NPLM_DWCONV_ESCRATCH and launch nothing. Every call on a GPU shares that GPU's array: two
  * calls that overlap in time on one GPU (different streams, or threads) race on it and corrupt each
  * other's dw/db; calls on one stream, or otherwise ordered, are safe. Nothing in the array has to be
