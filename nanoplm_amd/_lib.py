@@ -97,6 +97,8 @@ def load():
     lib.nplm_dwconv_bwd_tuned.restype = ctypes.c_int
     lib.nplm_dwconv_bwd_slabs.argtypes = [i64, i32, i32, i32, ctypes.POINTER(Tuning)]
     lib.nplm_dwconv_bwd_slabs.restype = i32
+    lib.nplm_dwconv_exec_kernel_size.argtypes = [i32]
+    lib.nplm_dwconv_exec_kernel_size.restype = i32
     lib.nplm_dwconv_debug_intervals.argtypes = [vp, i32, i64, i64, i64, i64, vp, vp]
     lib.nplm_dwconv_debug_intervals.restype = i64
     lib.nplm_dwconv_debug_copy.argtypes = [vp, vp, sz, vp]

@@ -1096,6 +1096,8 @@ size_t nplm_dwconv_bwd_workspace_bytes(int64_t T, int32_t C, int32_t K, int32_t 
     return (bytes + 255) & ~(size_t)255;
 }
 
+int32_t nplm_dwconv_exec_kernel_size(int32_t K) { return exec_kernel_size(K); }
+
 int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune) {
     if (check_common(T, C, K, 0, act_dtype, NPLM_DWCONV_F32) || T == 0) return 0;
     K = exec_kernel_size(K);

@@ -49,6 +49,8 @@ int nplm_dwconv_bwd_tuned(const void* x, const void* dy, const int32_t* cu, cons
 // Token-blocks (= workspace slabs of (K'+1)*C floats, K' the kernel size that runs: K, or for an odd K <= 31 without
 // kernels of its own the next of 3, 15, 31) a backward launch with these overrides uses.
 int32_t nplm_dwconv_bwd_slabs(int64_t T, int32_t C, int32_t K, int32_t act_dtype, const nplm_dwconv_tuning* tune);
+// The kernel size K' a plain or gated conv of K taps runs as (K itself for 3, 5, 7, 9, 15, 31 and above 31).
+int32_t nplm_dwconv_exec_kernel_size(int32_t K);
 
 // Host-side run of the kernels' boundary cursor (SeqCursor) over a HOST copy of cu: for rows
 // t = start, start+step, ... < T writes the interval [cs, ce) the cursor reports, located afresh

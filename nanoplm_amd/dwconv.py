@@ -121,11 +121,9 @@ def bwd_workspace_bytes(T: int, C: int, K: int, dtype: torch.dtype) -> int:
 
 
 def exec_kernel_size(K: int) -> int:
-    """The kernel size a plain conv of K taps runs as (csrc/dwconv_api.hip::exec_kernel_size): an odd K <= 31 that has no
-    kernels of its own takes the next size that has, with zero taps on either side; its dw/db slabs have that many rows."""
-    if K > 31 or K in (3, 5, 7, 9, 15, 31):
-        return K
-    return 3 if K < 3 else 15 if K < 15 else 31
+    """The kernel size a plain conv of K taps runs as: an odd K <= 31 that has no kernels of its own takes the next
+    size that has, with zero taps on either side; its dw/db slabs have that many rows."""
+    return int(_lib.load().nplm_dwconv_exec_kernel_size(K))
 
 
 def varlen_dwconv_bwd(x, dy, cu_seqlens, weight, *, need_dx=True, need_dw=True, residual: bool = False,
