@@ -52,21 +52,21 @@ VALU_PEAK_TFLOPS = 157.3  # MI355X fp32 vector ALU (256 CUs x 4 SIMDs x 32 FMA l
 # (workload name, kernel[, variant]). Counters cannot be read from inside this process, so a workload or variant
 # without an entry (configuration 1, --residual, other widths) reports traffic = null and says why.
 MEASURED_TRAFFIC = {
-    ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136263218,                       # 1.015 x algorithmic
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544056884,                   # 1.013 x
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816854701,                  # 1.014 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1076345885,       # 1.002 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619855210,      # 1.005 x
-    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272190087,    # 1.014 x
-    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410652860,   # 1.020 x
+    ("cfg2_bf16_fwd_T32768_C1024_K7", "forward"): 136261404,                       # 1.015 x algorithmic
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward"): 544057555,                   # 1.013 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward"): 816871634,                  # 1.014 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward"): 1075682217,       # 1.002 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward"): 1619868128,      # 1.005 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "forward"): 272198320,    # 1.014 x
+    ("cfg5_bf16_fwdbwd_T65536_C1024_K7_boundary_stress", "backward"): 410672393,   # 1.020 x
     # --gated --config 4 (profiles/bench_cfg4_gated_hbm_traffic.md)
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1635827018,    # 1.016 x
-    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693555429,   # 1.003 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "forward", "gated"): 1637482695,    # 1.016 x
+    ("cfg4_bf16_fwdbwd_T131072_C2048_K31_lognormal", "backward", "gated"): 2693567122,   # 1.003 x
     # --ln and --fp32 --ln (profiles/bench_cfg3_layernorm_fused_hbm_traffic.md); the backward figure is the fused kernel's alone
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551581056,             # 1.027 x
-    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830319410,            # 1.031 x
-    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "forward", "ln"): 1092089122,            # 1.017 x
-    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "backward", "ln"): 1641722624,           # 1.019 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "forward", "ln"): 551613338,             # 1.027 x
+    ("cfg3_bf16_fwdbwd_T131072_C1024_K7", "backward", "ln"): 830305929,            # 1.031 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "forward", "ln"): 1092201837,            # 1.017 x
+    ("cfg3_fp32_fwdbwd_T131072_C1024_K7", "backward", "ln"): 1641691951,           # 1.019 x
 }
 MIN_EVENT_LAUNCHES = 50   # per-kernel event samples, whatever --steps says
 
