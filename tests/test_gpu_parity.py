@@ -53,6 +53,28 @@ def test_configuration_matches_oracle(index):
     assert torch.equal(y, y2) and torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.equal(db, db2)
 
 
+@pytest.mark.parametrize("K", [11, 21])
+def test_headline_size_with_a_kernel_size_served_by_the_next_built_size(K):
+    """Configuration 3's tokens, lengths and width (T=131072, C=1024, bf16) with K = 11 (runs as 15) and K = 21 (runs as
+    31, the role-split kernels: every block walks 16 forward and 32 backward tiles) against the C oracle, and run twice."""
+    print(f"[case] configuration 3 with K={K}", flush=True)
+    wl = make_workload(3, with_dy=True)
+    g = torch.Generator().manual_seed(K)
+    w = (torch.randn(wl.C, K, generator=g) * K ** -0.5).bfloat16()
+    y64 = O.c_oracle_fwd(wl.x, wl.cu_seqlens, w, wl.bias)
+    dx64, dw64, db64 = O.c_oracle_bwd(wl.x, wl.dy, wl.cu_seqlens, w)
+    xd, dyd, cud, wd, bd = (t.to(DEV) for t in (wl.x, wl.dy, wl.cu_seqlens, w, wl.bias))
+    y = npa.varlen_dwconv_fwd(xd, cud, wd, bd)
+    dx, dw, db = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    assert dw.shape == (wl.C, K)
+    assert_act_close(y, y64, wl.dtype, f"K={K} y")
+    assert_act_close(dx, dx64, wl.dtype, f"K={K} dx")
+    assert_red_close(dw, dw64, f"K={K} dw")
+    assert_red_close(db, db64, f"K={K} db")
+    dx2, dw2, db2 = npa.varlen_dwconv_bwd(xd, dyd, cud, wd)
+    assert torch.equal(y, npa.varlen_dwconv_fwd(xd, cud, wd, bd)) and torch.equal(dx, dx2) and torch.equal(dw, dw2) and torch.equal(db, db2)
+
+
 def test_configuration_1_against_the_fp32_reference_path():
     """Configuration 1 is defined against the fp32 per-sequence conv1d path itself."""
     wl = make_workload(1)
