@@ -27,6 +27,47 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_header_is_plain_c_and_a_c_program_links_and_calls_the_library(tmp_path):
+    """include/nplm_dwconv.h compiles as strict C11 (no C++ left in it), every function it declares links from C against
+    the shared object, and a C caller gets the version, the error strings, the workspace size and the argument errors
+    (reported before anything is launched, so no GPU is needed)."""
+    import shutil
+    import subprocess
+    if shutil.which("gcc") is None:
+        pytest.skip("no C compiler")
+    header = open(os.path.join(ROOT, "include", "nplm_dwconv.h")).read()
+    names = sorted(set(re.findall(r"\b(nplm_dwconv_[a-z_]+)\s*\(", header)))
+    src = tmp_path / "abi.c"
+    src.write_text(
+        "#include <stdio.h>\n#include <string.h>\n#include \"nplm_dwconv.h\"\n"
+        "typedef void (*fn)(void);\n"
+        "int main(void) {\n"
+        "    fn all[] = {" + ", ".join(f"(fn){n}" for n in names) + "};\n"
+        "    char fake[64];\n"
+        "    void* a = (void*)(((size_t)fake + 15) & ~(size_t)15);   /* aligned, never dereferenced */\n"
+        "    if (sizeof(all) / sizeof(all[0]) != " + str(len(names)) + ") return 10;\n"
+        "    if (nplm_dwconv_version() < 100) return 11;\n"
+        "    if (strcmp(nplm_dwconv_strerror(0), \"success\") != 0) return 12;\n"
+        "    if (!strstr(nplm_dwconv_strerror(-NPLM_DWCONV_EKSIZE), \"odd\")) return 13;\n"
+        "    if (nplm_dwconv_fwd(NULL, a, a, a, a, 128, 64, 3, 1, NPLM_DWCONV_BF16, NPLM_DWCONV_BF16, NULL) != -NPLM_DWCONV_ENULL) return 14;\n"
+        "    if (nplm_dwconv_fwd(a, a, a, a, a, 128, 64, 4, 1, NPLM_DWCONV_BF16, NPLM_DWCONV_BF16, NULL) != -NPLM_DWCONV_EKSIZE) return 15;\n"
+        "    if (nplm_dwconv_bwd(a, a, a, a, a, a, a, NULL, 0, 128, 64, 3, 1, NPLM_DWCONV_F32, NPLM_DWCONV_F32, NULL) != -NPLM_DWCONV_EWORKSPACE) return 16;\n"
+        "    if (nplm_dwconv_fwd(NULL, NULL, NULL, NULL, NULL, 0, 64, 3, 0, NPLM_DWCONV_F32, NPLM_DWCONV_F32, NULL) != 0) return 17;   /* empty batch */\n"
+        "    printf(\"%zu %zu\\n\", nplm_dwconv_bwd_workspace_bytes(131072, 1024, 7, NPLM_DWCONV_BF16), nplm_dwconv_bwd_workspace_bytes(131072, 1024, 11, NPLM_DWCONV_BF16));\n"
+        "    return 0;\n}\n")
+    exe = tmp_path / "abi"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    cc = subprocess.run(["gcc", "-std=c11", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),
+                         str(src), "-o", str(exe), "-L", libdir, "-l:" + os.path.basename(_lib.LIB_PATH), "-Wl,-rpath," + libdir,
+                         "-Wl,-rpath-link,/opt/rocm/lib"], capture_output=True, text=True)
+    assert cc.returncode == 0, cc.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert run.returncode == 0, (run.returncode, run.stderr)
+    lib = _lib.load()
+    want = f"{lib.nplm_dwconv_bwd_workspace_bytes(131072, 1024, 7, 1)} {lib.nplm_dwconv_bwd_workspace_bytes(131072, 1024, 11, 1)}"
+    assert run.stdout.strip() == want
+
+
 def test_version_and_strerror():
     lib = _lib.load()
     assert lib.nplm_dwconv_version() >= 100
