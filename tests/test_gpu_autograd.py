@@ -170,3 +170,30 @@ def test_forward_and_backward_replay_correctly_from_a_hip_graph():
         torch.cuda.synchronize()
         assert torch.equal(gy, ey) and torch.equal(gdx, edx), f"replay {it}"
         assert torch.equal(gdw, edw) and torch.equal(gdb, edb), f"replay {it}"
+
+
+def test_the_integration_guides_ctypes_binding_runs_as_written():
+    """The reference-side binding a maintainer would paste (the first Python block of the integration guide: a ctypes
+    load of the shared object and an autograd Function over the two plain entry points) is executed as it stands, with
+    only the library's file name replaced by its path, and gives this package's own results bit for bit."""
+    import os
+    import re
+    from nanoplm_amd import _lib
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    guide = open(os.path.join(root, "INTEGRATION.md")).read()
+    block = re.search(r"```python\n(import ctypes, torch\n.*?)```", guide, re.S).group(1)
+    assert 'ctypes.CDLL("libnplm_dwconv.so")' in block
+    ns = {}
+    exec(block.replace('"libnplm_dwconv.so"', repr(_lib.LIB_PATH)), ns)
+    fn = ns["VarlenDWConv1dFunction"]
+    for cfg, kw in ((1, {}), (5, dict(T=5000, C=512))):
+        wl = make_workload(cfg, with_dy=True, **kw)
+        d = wl.to(DEV)
+        x = d.x.clone().requires_grad_(True)
+        w = d.weight.clone().requires_grad_(True)
+        b = d.bias.clone().requires_grad_(True)
+        y = fn.apply(x, d.cu_seqlens, w, b)
+        y.backward(d.dy)
+        assert torch.equal(y, npa.varlen_dwconv_fwd(d.x, d.cu_seqlens, d.weight, d.bias))
+        dx, dw, db = npa.varlen_dwconv_bwd(d.x, d.dy, d.cu_seqlens, d.weight)
+        assert torch.equal(x.grad, dx) and torch.equal(w.grad, dw.to(w.dtype)) and torch.equal(b.grad, db.to(b.dtype))
